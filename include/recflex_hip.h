@@ -1,0 +1,154 @@
+/*
+ * C ABI of the MI355X (gfx950) fused-embedding path.
+ *
+ * Two kinds of shared library implement it:
+ *
+ *  1. librecom.so -- one per emitted model (the code emitter writes process.hip, hipcc builds
+ *     it).  It holds the fused kernel `FusedKnl` specialised to the model's feature list and
+ *     exports the recom_* entry points below.  It replaces the reference's generated torch
+ *     extension (TORCH_LIBRARY(recom): RecFlex/code_emitter/codegen.py:454-461).
+ *     Several such libraries can be loaded into one process (dlopen / ctypes.CDLL), each
+ *     with its own handle.
+ *
+ *  2. librecflex_host.so -- model independent, CPU only.  It exports the recom_host_* entry
+ *     points: the text front end that turns the reference's dataset lines into indices and
+ *     offsets and packs them.  It replaces the generated pybind module `recom_host`
+ *     (RecFlex/code_emitter/codegen.py:90-218) and the per-schedule string parsers
+ *     (examples/csrc/{warp_per_sample,one_block_multi_sample,onehot}_preprocess.cu).
+ *
+ * All functions return 0 on success.  recom_* functions return the hipError_t of the first
+ * failing HIP call otherwise (never exit(), never synchronise the device, never allocate or
+ * free device memory); recom_host_* functions return a negative RECOM_HOST_E* code.
+ * Plain pointers and sizes only: no torch types cross this boundary.
+ */
+#ifndef RECFLEX_HIP_H_
+#define RECFLEX_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * librecom.so (generated, GPU)
+ * ---------------------------------------------------------------------------------------- */
+
+/* table element types (MetaData.data_type: "float", "half", "int8") */
+#define RECOM_DTYPE_F32 0
+#define RECOM_DTYPE_F16 1
+/* row = dim unsigned 8-bit codes + fp16 scale + fp16 bias, row stride rounded up to 16 B;
+ * value = code * scale + bias */
+#define RECOM_DTYPE_I8 2
+
+typedef struct recom_info {
+  int32_t abi_version;    /* RECOM_ABI_VERSION */
+  int32_t num_features;   /* F */
+  int32_t embed_dim_sum;  /* columns of the pooled output */
+  int32_t block_threads;  /* workgroup size the kernel was emitted for */
+  int32_t occupancy;      /* workgroups per CU the kernel was emitted for (0 = not limited) */
+  int32_t num_bodies;     /* distinct schedule bodies after de-duplication */
+  int32_t timing;         /* 1 if built with per-feature device timers */
+  int32_t tile_bytes;     /* default memory traffic per tile used by the run-time binding */
+  int32_t static_binding; /* 1 if the tile count per feature was fixed at emit time */
+  int32_t reserved[7];
+} recom_info;
+
+#define RECOM_ABI_VERSION 1
+
+/* Static description of the emitted kernel.  No reference counterpart as a function: the
+ * reference bakes the same numbers into process.cu (EMBED_DIM_SUM, block_threads,
+ * RecFlex/code_emitter/codegen.py:227-231,318-319). */
+int recom_get_info(recom_info *out);
+
+/* Per-feature static tables, each `num_features` long; any pointer may be NULL.
+ * embed_dims / embed_dim_offsets: RecFlex/code_emitter/codegen.py:227-231,289-292
+ * (d_embed_dim_offsets).  dtypes: RECOM_DTYPE_*.  row_strides: bytes between table rows. */
+int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_offsets, int32_t *dtypes,
+                             int32_t *row_strides);
+
+/* Workgroups of FusedKnl that are resident at once on the current device
+ * (= CUs x workgroups per CU at the emitted occupancy); this is also the size of the
+ * persistent grid.  Replaces torch.ops.recom.get_max_concurrent_blocks
+ * (RecFlex/code_emitter/codegen.py:446-452, RecFlex/sched_basic_csrc/include/utils.cuh:6-21). */
+int recom_get_max_concurrent_blocks(int32_t *out);
+
+typedef struct recom_process_args {
+  /* device int64[F]: base address of each feature's table
+   * (RecFlex/sched_basic_csrc/gpu_pointers_array.cc:16-25) */
+  const int64_t *d_embed_table_ptrs;
+  /* Input, form A: device int64[2F], [2f] = address of feature f's int32 indices[L_f],
+   * [2f+1] = address of its int32 offsets[batch+1].  NULL selects form B. */
+  const int64_t *d_io_ptrs;
+  /* Input, form B (the packed buffer of RecFlex/rec_modules.py:40-42): feature f's data
+   * start at d_arg_buffers + d_arg_buffer_offsets[f] (bytes, device int64[F+1]):
+   * int32 offsets[batch+1], padded to 128 B, then int32 indices[L_f], padded to 128 B. */
+  const void *d_arg_buffers;
+  const int64_t *d_arg_buffer_offsets;
+  /* device fp32 [batch, embed_dim_sum], row-major, caller allocated; every element is
+   * written (empty bag -> zeros).  The reference allocates it inside the op
+   * (RecFlex/code_emitter/codegen.py:416-421). */
+  float *d_output;
+  int32_t batch;
+  /* memory traffic per tile for the run-time binding; 0 = the emitted default */
+  int32_t tile_bytes;
+  /* persistent grid size; 0 = recom_get_max_concurrent_blocks() */
+  int32_t grid_blocks;
+  /* timing builds only: device uint64[F], the kernel ADDS each feature's workgroup-ticks
+   * (s_memtime) to it; caller zeroes it.  Replaces the per-block clock() array
+   * (RecFlex/code_emitter/codegen.py:301-316,388-401).  Must be NULL otherwise. */
+  unsigned long long *d_times;
+  /* hipStream_t to launch on (NULL = the null stream) */
+  void *stream;
+} recom_process_args;
+
+/* Launch the fused kernel: for every feature f and sample b,
+ *   output[b, off_f : off_f + D_f] = sum_{p in [offsets_f[b], offsets_f[b+1])} row(table_f, indices_f[p])
+ * Asynchronous.  Replaces torch.ops.recom.process (RecFlex/code_emitter/codegen.py:403-444)
+ * and FusedKnl (RecFlex/code_emitter/codegen.py:318-383). */
+int recom_process(const recom_process_args *args);
+
+/* ------------------------------------------------------------------------------------------
+ * librecflex_host.so (CPU)
+ * ---------------------------------------------------------------------------------------- */
+
+#define RECOM_HOST_EINVAL (-1)   /* NULL pointer / negative size */
+#define RECOM_HOST_ENOSPC (-2)   /* output capacity too small */
+#define RECOM_HOST_ELINES (-3)   /* text holds a different number of lines than expected */
+#define RECOM_HOST_ERANGE (-4)   /* value does not fit in int32 */
+
+/* Parse `num_lines` '\n'-separated sample lines of one feature.  Inside a line any byte that
+ * is not a decimal digit separates two indices and a non-empty line always ends an index, so
+ * "3,,5" gives 3,0,5 and "" gives an empty bag
+ * (examples/csrc/warp_per_sample_preprocess.cu:14-32; the one-hot parser
+ * examples/csrc/onehot_preprocess.cu:9-11 is the single-index case).
+ * offsets_out[num_lines+1] receives the exclusive prefix sum of the bag lengths,
+ * indices_out[0..*num_indices_out) the indices.  A final '\n' after the last line is allowed. */
+int recom_host_parse_lines(const char *text, int64_t text_len, int32_t num_lines,
+                           int32_t *indices_out, int64_t indices_capacity,
+                           int32_t *offsets_out, int64_t *num_indices_out);
+
+/* Upper bound of the number of indices a text of this length can hold. */
+int64_t recom_host_max_indices(int64_t text_len);
+
+/* 128-byte alignment used inside the packed argument buffer
+ * (RecFlex/sched_basic_csrc/include/utils.cuh:60-68). */
+int64_t recom_host_alignmem(int64_t nbytes);
+
+/* Bytes feature f occupies in the packed buffer (form B above). */
+int64_t recom_host_packed_size(int32_t batch, int64_t num_indices);
+
+/* Pack F features into form B.  offsets[f] -> int32[batch+1], indices[f] -> int32[n_f].
+ * dst has room for dst_capacity bytes; byte_offsets_out[F+1] receives each feature's start
+ * (RecFlex/code_emitter/codegen.py:149-160 computes the same offsets for the reference's
+ * layout).  Padding bytes are zeroed. */
+int recom_host_pack(int32_t num_features, int32_t batch, const int32_t *const *offsets,
+                    const int32_t *const *indices, const int64_t *num_indices, void *dst,
+                    int64_t dst_capacity, int64_t *byte_offsets_out);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* RECFLEX_HIP_H_ */

@@ -1,0 +1,435 @@
+"""Feature-specific schedule fusion for gfx950: emits ``process.hip`` (the fused kernel
+``FusedKnl`` plus its C-ABI entry points), ``preprocess.cpp`` (the host text front end) and a
+``CMakeLists.txt`` that builds both with hipcc / g++.
+
+Keeps the interface of the reference's ``CodeEmitter``
+(``RecFlex/code_emitter/codegen.py:20-568``: ``emit``, ``emit_host``, ``emit_cmake_list``,
+``serialize_config``, ``emit_if_updated``, de-duplication of identical schedule bodies
+``:233-243``, per-feature ``__device__`` tables ``:279-299``, in-kernel timers ``:301-316``).
+What is emitted is new:
+
+* The kernel is a persistent grid.  Every workgroup computes the thread binding itself from
+  the live offsets (``rfx::bind_tiles``), then walks the tile space with stride ``gridDim.x``
+  and dispatches each tile to its feature's schedule body through a ``switch`` (``inline``)
+  or through calls to ``__noinline__`` functions.  There is no host-built task mapping.
+* Entry points are plain C (``include/recflex_hip.h``), loaded with ``ctypes``; several
+  emitted libraries can live in one process.
+* Timing builds add each tile's ``s_memtime`` ticks to a per-feature accumulator instead of
+  storing one stamp per block.
+"""
+
+import json
+import os
+from typing import Any, Dict, List, NamedTuple, Optional, Tuple
+
+from .schedule_base import ScheduleBase, ScheduleVars, PreprocessVars
+from .build_basic import BasicBuilder
+
+# memory traffic (bytes) the run-time binding aims at per tile
+DEFAULT_TILE_BYTES = 64 * 1024
+# per-bag traffic that does not depend on the bag length, besides the output slice: one offset
+BAG_FIXED_BYTES = 4
+INDEX_BYTES = 4
+
+
+def _c_array(ctype: str, name: str, values: List[int], per_line: int = 16) -> str:
+    lines = []
+    for i in range(0, len(values), per_line):
+        lines.append("    " + ", ".join(str(v) for v in values[i:i + per_line]))
+    body = ",\n".join(lines) if lines else "    0"
+    return f"__constant__ {ctype} {name}[] = {{\n{body}\n}};\n\n"
+
+
+class CodeEmitter:
+    def __init__(self, feat_schedules: List[Tuple[ScheduleBase, NamedTuple]]):
+        self.feat_schedules: List[Tuple[ScheduleBase, NamedTuple]] = feat_schedules
+        if len(self.feat_schedules) > 0:
+            self.block_threads: int = feat_schedules[0][0].block_threads
+            for schedule, params in feat_schedules:
+                assert self.block_threads == schedule.block_threads
+
+    # ------------------------------------------------------------------ configuration dump
+
+    def serialize_config(self) -> List[Dict[str, Any]]:
+        return [
+            {
+                "schedule": schedule.__class__.__name__,
+                "params": params._asdict(),
+                "embed_dim": schedule.meta.embed_dim,
+                "data_type": schedule.meta.data_type,
+            }
+            for schedule, params in self.feat_schedules
+        ]
+
+    def dump_key(self, fname: str) -> None:
+        with open(fname, "w") as f:
+            json.dump(self.serialize_config(), fp=f, indent=1)
+
+    # ------------------------------------------------------------------ derived tables
+
+    def embed_dims(self) -> List[int]:
+        return [sched.meta.embed_dim for sched, _ in self.feat_schedules]
+
+    def embed_dim_offsets(self) -> List[int]:
+        offsets = [0]
+        for d in self.embed_dims():
+            offsets.append(offsets[-1] + d)
+        return offsets
+
+    def out_vec(self) -> int:
+        """Widest output store (floats) that is aligned for every feature's column offset."""
+        offs = self.embed_dim_offsets()
+        for w in (4, 2):
+            if all(o % w == 0 for o in offs):
+                return w
+        return 1
+
+    def dedup(self) -> Tuple[Dict[int, int], List[int]]:
+        """feature -> id of the first feature with the same (LDS type, body); list of those ids."""
+        seen: Dict[str, int] = {}
+        id_map: Dict[int, int] = {}
+        for feat_idx, (schedule, params) in enumerate(self.feat_schedules):
+            key = schedule.EmitShmemType(params) + "\n" + schedule.EmitScheduleBody(params)
+            if key not in seen:
+                seen[key] = feat_idx
+            id_map[feat_idx] = seen[key]
+        return id_map, list(seen.values())
+
+    # ------------------------------------------------------------------ device code
+
+    def emit_headers(self) -> str:
+        headers = {"<hip/hip_runtime.h>", "<stdint.h>", '"recflex_hip.h"', '"rfx_binding.hip.h"',
+                   '"rfx_launch.hip.h"'}
+        for schedule, params in self.feat_schedules:
+            headers = headers.union(schedule.EmitHeaders())
+        return ''.join(sorted(f"#include {header}\n" for header in headers)) + '\n'
+
+    def emit_kernel(self, occupancy: int = None, inline: bool = True, timing: bool = False,
+                    timing_branch: bool = False, fixed_task_block_nums: List[int] = None,
+                    tile_bytes: int = None) -> str:
+        num_feats = len(self.feat_schedules)
+        assert num_feats > 0, "cannot emit a fused kernel for zero features"
+        vars_ = ScheduleVars()
+        id_map, body_ids = self.dedup()
+        embed_dim_offsets = self.embed_dim_offsets()
+
+        consts = f'''constexpr int NUM_FEATS = {num_feats};
+constexpr int {vars_.EMBED_DIM_SUM} = {embed_dim_offsets[-1]};
+constexpr int {vars_.BLOCK_THREADS} = {self.block_threads};
+constexpr int {vars_.out_vec} = {self.out_vec()};
+constexpr int OCCUPANCY = {occupancy if occupancy else 0};
+constexpr int TILE_BYTES = {tile_bytes if tile_bytes else DEFAULT_TILE_BYTES};
+constexpr int NUM_BODIES = {len(body_ids)};
+constexpr bool TIMING = {"true" if timing else "false"};
+constexpr bool STATIC_BINDING = {"true" if fixed_task_block_nums else "false"};
+
+'''
+
+        temp_storage_decl = "union KnlTempStorage {\n"
+        functions = ""
+        for feat_idx in body_ids:
+            schedule, params = self.feat_schedules[feat_idx]
+            temp_storage_decl += f"  {schedule.EmitShmemType(params)} f{feat_idx};\n"
+            functions += f'''
+__device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{feat_idx}(
+    const char *__restrict__ {vars_.embed_table},
+    const int *__restrict__ {vars_.indices},
+    const int *__restrict__ {vars_.offsets},
+    float *__restrict__ {vars_.output},
+    const int {vars_.embed_dim_offset},
+    const int {vars_.bag_begin}, const int {vars_.bag_end},
+    char *__restrict__ {vars_.shmem}) {{
+  {schedule.EmitScheduleBody(params)}
+}}
+'''
+        temp_storage_decl += "};\n\n"
+
+        tables = _c_array("int", "c_process_func_ids", [id_map[f] for f in range(num_feats)])
+        tables += _c_array("int", "c_embed_dim_offsets", embed_dim_offsets)
+        tables += _c_array("int", "c_lookup_bytes",
+                           [s.meta.row_bytes + INDEX_BYTES for s, _ in self.feat_schedules])
+        tables += _c_array("int", "c_bag_bytes",
+                           [s.meta.embed_dim * 4 + BAG_FIXED_BYTES for s, _ in self.feat_schedules])
+        tables += _c_array("int", "c_tile_gran",
+                           [s.TileGranularity(p) for s, p in self.feat_schedules])
+        if fixed_task_block_nums:
+            assert len(fixed_task_block_nums) == num_feats
+            tables += _c_array("int", "c_fixed_task_block_nums",
+                               [max(1, int(n)) for n in fixed_task_block_nums])
+
+        timing_begin = '''
+    __syncthreads();
+    const unsigned long long t_begin = __builtin_amdgcn_s_memtime();
+''' if timing else ''
+        timing_end = '''
+    __syncthreads();
+    if (threadIdx.x == 0)
+      atomicAdd(&d_times[feat_idx], __builtin_amdgcn_s_memtime() - t_begin);
+''' if timing else ''
+
+        call_args = (f"table, indices, offsets, d_output, embed_dim_offset, "
+                     f"{vars_.bag_begin}, {vars_.bag_end}, reinterpret_cast<char *>(&s)")
+        cases = "".join(
+            f"      case {feat_idx}: ProcessFeat{feat_idx}({call_args}); break;\n"
+            for feat_idx in body_ids)
+
+        launch_bounds = (f"__launch_bounds__({vars_.BLOCK_THREADS}, {occupancy})" if occupancy
+                         else f"__launch_bounds__({vars_.BLOCK_THREADS})")
+        kernel = f'''
+extern "C" __global__ void {launch_bounds} FusedKnl(
+    const int64_t *__restrict__ d_embed_table_ptrs,
+    const int64_t *__restrict__ d_io_ptrs,
+    const char *__restrict__ d_arg_buffers,
+    const int64_t *__restrict__ d_arg_buffer_offsets,
+    float *__restrict__ d_output,
+    const int batch, const int tile_bytes,
+    unsigned long long *__restrict__ d_times) {{
+  __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;
+  __shared__ KnlTempStorage s;
+
+  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
+  const int total_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}>(
+      s_bind, io, tile_bytes, c_lookup_bytes, c_bag_bytes, c_tile_gran,
+      {"c_fixed_task_block_nums" if fixed_task_block_nums else "nullptr"});
+
+  for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {{
+{timing_begin if timing and timing_branch else ''}
+    const int feat_idx = __builtin_amdgcn_readfirstlane(rfx::find_feature<NUM_FEATS>(s_bind, tile));
+    const int bags_per_tile = s_bind.bags_per_tile[feat_idx];
+    const int {vars_.bag_begin} = (tile - s_bind.prefix[feat_idx]) * bags_per_tile;
+    const int {vars_.bag_end} = min(batch, {vars_.bag_begin} + bags_per_tile);
+    const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[feat_idx]);
+    const int *indices = io.indices(feat_idx);
+    const int *offsets = io.offsets(feat_idx);
+    const int embed_dim_offset = c_embed_dim_offsets[feat_idx];
+{timing_begin if timing and not timing_branch else ''}
+    switch (c_process_func_ids[feat_idx]) {{
+{cases}      default: break;
+    }}
+{timing_end}
+  }}
+}}
+
+'''
+        return consts + temp_storage_decl + functions + "\n" + tables + kernel
+
+    def emit_process_func(self, timing: bool = False, occupancy: int = None) -> str:
+        return '''
+extern "C" int recom_process(const recom_process_args *a) {
+  if (!a || !a->d_embed_table_ptrs || !a->d_output || a->batch < 0 ||
+      (!a->d_io_ptrs && (!a->d_arg_buffers || !a->d_arg_buffer_offsets)))
+    return static_cast<int>(hipErrorInvalidValue);
+  if (TIMING != (a->d_times != nullptr)) return static_cast<int>(hipErrorInvalidValue);
+  if (a->tile_bytes < 0 || a->grid_blocks < 0) return static_cast<int>(hipErrorInvalidValue);
+  if (a->batch == 0) return static_cast<int>(hipSuccess);
+
+  const rfx::LaunchState *st = nullptr;
+  hipError_t e = rfx::get_launch_state(FusedKnl, BLOCK_THREADS, OCCUPANCY, &st);
+  if (e != hipSuccess) return static_cast<int>(e);
+  const int grid = a->grid_blocks > 0 ? a->grid_blocks : st->cus * st->occupancy;
+  if (grid <= 0) return static_cast<int>(hipErrorInvalidConfiguration);
+  const int tile_bytes = a->tile_bytes > 0 ? a->tile_bytes : TILE_BYTES;
+
+  hipLaunchKernelGGL(FusedKnl, dim3(grid), dim3(BLOCK_THREADS), st->dyn_lds,
+                     static_cast<hipStream_t>(a->stream),
+                     a->d_embed_table_ptrs, a->d_io_ptrs,
+                     static_cast<const char *>(a->d_arg_buffers), a->d_arg_buffer_offsets,
+                     a->d_output, a->batch, tile_bytes, a->d_times);
+  return static_cast<int>(hipGetLastError());
+}
+'''
+
+    def emit_get_concurrent_blocks_func(self, occupancy: int = None) -> str:
+        return '''
+extern "C" int recom_get_max_concurrent_blocks(int32_t *out) {
+  if (!out) return static_cast<int>(hipErrorInvalidValue);
+  const rfx::LaunchState *st = nullptr;
+  hipError_t e = rfx::get_launch_state(FusedKnl, BLOCK_THREADS, OCCUPANCY, &st);
+  if (e != hipSuccess) return static_cast<int>(e);
+  *out = st->cus * st->occupancy;
+  return static_cast<int>(hipSuccess);
+}
+'''
+
+    def emit_process_ops(self) -> str:
+        return '''
+extern "C" int recom_get_info(recom_info *out) {
+  if (!out) return static_cast<int>(hipErrorInvalidValue);
+  *out = recom_info{};
+  out->abi_version = RECOM_ABI_VERSION;
+  out->num_features = NUM_FEATS;
+  out->embed_dim_sum = EMBED_DIM_SUM;
+  out->block_threads = BLOCK_THREADS;
+  out->occupancy = OCCUPANCY;
+  out->num_bodies = NUM_BODIES;
+  out->timing = TIMING ? 1 : 0;
+  out->tile_bytes = TILE_BYTES;
+  out->static_binding = STATIC_BINDING ? 1 : 0;
+  return 0;
+}
+
+// host copies of the per-feature tables (the __constant__ arrays above are device symbols)
+static const int h_embed_dims[] = {H_EMBED_DIMS};
+static const int h_embed_dim_offsets[] = {H_EMBED_DIM_OFFSETS};
+static const int h_dtypes[] = {H_DTYPES};
+static const int h_row_strides[] = {H_ROW_STRIDES};
+
+extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_offsets,
+                                        int32_t *dtypes, int32_t *row_strides) {
+  for (int f = 0; f < NUM_FEATS; ++f) {
+    if (embed_dims) embed_dims[f] = h_embed_dims[f];
+    if (embed_dim_offsets) embed_dim_offsets[f] = h_embed_dim_offsets[f];
+    if (dtypes) dtypes[f] = h_dtypes[f];
+    if (row_strides) row_strides[f] = h_row_strides[f];
+  }
+  return 0;
+}
+'''.replace("H_EMBED_DIMS", ", ".join(map(str, self.embed_dims()))) \
+   .replace("H_EMBED_DIM_OFFSETS", ", ".join(map(str, self.embed_dim_offsets()[:-1]))) \
+   .replace("H_DTYPES", ", ".join(str(s.meta.dtype_id) for s, _ in self.feat_schedules)) \
+   .replace("H_ROW_STRIDES", ", ".join(str(s.meta.row_stride) for s, _ in self.feat_schedules))
+
+    # ------------------------------------------------------------------ files
+
+    def emit_if_updated(self, fname: str, code: str) -> bool:
+        if os.path.exists(fname):
+            with open(fname) as f:
+                old = f.read()
+                if old.strip() == code.strip():
+                    return False
+
+        with open(fname, "w") as f:
+            f.write(code)
+        return True
+
+    def emit(self, ofname: str, occupancy: int = None, inline: bool = True,
+             tune: bool = False, timing: bool = False, timing_branch: bool = False,
+             fixed_task_block_nums: List[int] = None, tile_bytes: int = None) -> None:
+        """Write the device source.  ``occupancy`` = workgroups per CU the kernel is built and
+        launched for (``__launch_bounds__`` budget, persistent grid size, and a dynamic-LDS pad
+        that keeps further workgroups off the CU); ``tune`` is accepted for signature
+        compatibility -- the pad is applied whenever an occupancy is given."""
+        code = "// generated by recflex_amd.code_emitter -- do not edit\n"
+        code += self.emit_headers()
+        code += self.emit_kernel(timing=timing, timing_branch=timing_branch,
+                                 occupancy=occupancy, inline=inline,
+                                 fixed_task_block_nums=fixed_task_block_nums,
+                                 tile_bytes=tile_bytes)
+        code += self.emit_process_func(timing=timing, occupancy=occupancy)
+        code += self.emit_get_concurrent_blocks_func(occupancy=occupancy)
+        code += self.emit_process_ops()
+
+        self.emit_if_updated(ofname, code)
+
+    def emit_host_op_headers(self) -> str:
+        headers = {"<stdint.h>"}
+        for schedule, params in self.feat_schedules:
+            headers = headers.union(schedule.EmitPrepropHeaders())
+        return ''.join(sorted(f"#include {header}\n" for header in headers)) + '\n'
+
+    def emit_host_preprocess(self, fixed_task_block_nums: List[int] = None) -> str:
+        num_feats = len(self.feat_schedules)
+        v = PreprocessVars()
+        seen: Dict[str, int] = {}
+        id_map: Dict[int, int] = {}
+        functions = ""
+        for feat_idx, (schedule, params) in enumerate(self.feat_schedules):
+            snippet = schedule.EmitHostPreprocess(params)
+            if snippet not in seen:
+                seen[snippet] = feat_idx
+                functions += f'''
+static int PreprocFeat{feat_idx}(
+    const char *{v.raw_data}, const int64_t {v.raw_data_len}, const int32_t {v.num_lines},
+    int32_t *{v.indices}, const int64_t {v.indices_capacity}, int32_t *{v.offsets},
+    int64_t *{v.num_inputs_ref}) {{
+{snippet}}}
+'''
+            id_map[feat_idx] = seen[snippet]
+
+        table = ",\n".join(f"    PreprocFeat{id_map[f]}" for f in range(num_feats))
+        dims = ", ".join(map(str, self.embed_dims()))
+        return functions + f'''
+typedef int (*PreprocFeatT)(const char *, const int64_t, const int32_t, int32_t *,
+                            const int64_t, int32_t *, int64_t *);
+static const PreprocFeatT preproc_feats[] = {{
+{table}
+}};
+static const int32_t embed_dims[] = {{{dims}}};
+
+extern "C" int32_t recom_host_num_features() {{ return {num_feats}; }}
+
+// bytes of one pooled output row of feature `feat`
+extern "C" int64_t recom_host_output_row_bytes(int32_t feat) {{
+  return feat >= 0 && feat < {num_feats} ? int64_t(embed_dims[feat]) * 4 : -1;
+}}
+
+// parse the '\\n'-joined sample lines of feature `feat`
+extern "C" int recom_host_preprocess_feat(
+    int32_t feat, const char *{v.raw_data}, int64_t {v.raw_data_len}, int32_t {v.num_lines},
+    int32_t *{v.indices}, int64_t {v.indices_capacity}, int32_t *{v.offsets},
+    int64_t *{v.num_inputs_ref}) {{
+  if (feat < 0 || feat >= {num_feats}) return RECOM_HOST_EINVAL;
+  return preproc_feats[feat]({v.raw_data}, {v.raw_data_len}, {v.num_lines}, {v.indices},
+                             {v.indices_capacity}, {v.offsets}, {v.num_inputs_ref});
+}}
+'''
+
+    def emit_host(self, ofname: str, fixed_task_block_nums: List[int] = None) -> None:
+        code = "// generated by recflex_amd.code_emitter -- do not edit\n"
+        code += self.emit_host_op_headers()
+        code += self.emit_host_preprocess(fixed_task_block_nums=fixed_task_block_nums)
+        self.emit_if_updated(ofname, code)
+
+    def emit_cmake_list(self, ofname: str, code_fname: str, host_fname: str,
+                        subdirs: List[str] = [], includes: List[str] = [],
+                        links: List[str] = [], host_links: List[str] = [],
+                        extra: str = "", debug: bool = False) -> None:
+        """CMake project (no compiled languages enabled) whose targets run hipcc for
+        ``librecom.so`` and g++ for ``recom_host.so``; ``cmake .. && make`` in ``build/``
+        produces both, as with the reference's generated CMakeLists.txt (codegen.py:489-568)."""
+        basic = BasicBuilder()
+        includes = list(includes) + [basic.include, basic.abi_include]
+        inc_flags = " ".join(f"-I{inc}" for inc in includes)
+        link_flags = " ".join(links)
+        host_link_flags = " ".join(host_links)
+        opt = "-g -O0" if debug else "-O3"
+        add_subdirs = '\n'.join(f"add_subdirectory({subdir})" for subdir in subdirs)
+
+        recom = f'''
+add_custom_command(
+  OUTPUT ${{CMAKE_BINARY_DIR}}/librecom.so
+  COMMAND {basic.hipcc} {" ".join(basic.hip_flags)} {opt} {inc_flags}
+          ${{CMAKE_SOURCE_DIR}}/{code_fname} {link_flags} -o ${{CMAKE_BINARY_DIR}}/librecom.so
+  DEPENDS ${{CMAKE_SOURCE_DIR}}/{code_fname}
+  VERBATIM)
+add_custom_target(recom ALL DEPENDS ${{CMAKE_BINARY_DIR}}/librecom.so)
+''' if code_fname else ''
+
+        recom_host = f'''
+add_custom_command(
+  OUTPUT ${{CMAKE_BINARY_DIR}}/recom_host.so
+  COMMAND {basic.cxx} {" ".join(basic.host_flags)} {opt} {inc_flags}
+          ${{CMAKE_SOURCE_DIR}}/{host_fname} {basic.host_source} {host_link_flags}
+          -o ${{CMAKE_BINARY_DIR}}/recom_host.so
+  DEPENDS ${{CMAKE_SOURCE_DIR}}/{host_fname} {basic.host_source}
+  VERBATIM)
+add_custom_target(recom_host ALL DEPENDS ${{CMAKE_BINARY_DIR}}/recom_host.so)
+''' if host_fname else ''
+
+        code = f'''
+cmake_minimum_required(VERSION 3.12 FATAL_ERROR)
+project(recom_project LANGUAGES NONE)
+
+# Add subdirectories
+{add_subdirs}
+
+# Add target recom_host
+{recom_host}
+
+# Add target recom
+{recom}
+
+# Extra area
+{extra}
+'''
+        self.emit_if_updated(ofname, code)

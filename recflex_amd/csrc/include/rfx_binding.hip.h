@@ -1,0 +1,130 @@
+// Run-time thread binding of the fused embedding kernel, computed on the device.
+//
+// Every workgroup of the persistent grid derives, from the live offsets of the batch, how many
+// tiles (ranges of consecutive bags worth about `tile_bytes` of memory traffic) each feature
+// gets, exclusive-scans these counts in LDS and then walks the global tile space
+// [0, total_tiles) with stride gridDim.x, finding the owning feature of a tile by binary search
+// in the LDS prefix array.  A feature with long bags therefore gets many small bag ranges, a
+// feature with short bags few large ones, and no host-side mapping or read-back is needed.
+//
+// Reference counterparts: the host-built (feature, block) list GetTaskMapping
+// (RecFlex/sched_basic_csrc/task_mapping.cu:6-18), the per-feature num_tiles/num_blocks
+// computed in the host preprocessors (examples/csrc/warp_per_sample_preprocess.cu:34-37) and
+// the lookup `d_task_mapping[blockIdx.x]` at the top of the generated kernel
+// (RecFlex/code_emitter/codegen.py:331-336).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rfx {
+
+// A device address read from memory, as a pointer the compiler knows to be global memory (so
+// that accesses become global_load/global_store instead of flat ones).
+template <typename T> __device__ __forceinline__ const T *global_ptr(int64_t addr) {
+  typedef const T __attribute__((address_space(1))) * gptr_t;
+  return (const T *)reinterpret_cast<gptr_t>(addr);
+}
+
+// 128-byte alignment of the vectors inside a packed argument buffer
+// (RecFlex/sched_basic_csrc/include/utils.cuh:60-62)
+__host__ __device__ constexpr int64_t alignmem(int64_t x) { return (x + 127) / 128 * 128; }
+
+// Where a feature's int32 offsets[batch+1] and indices[] live.  Two forms are accepted:
+//  * pointer table: io_ptrs[2f] = indices, io_ptrs[2f+1] = offsets (device addresses);
+//  * packed buffer: feature f starts at arg_base + arg_offsets[f] (bytes) with its offsets,
+//    padded to 128 B, followed by its indices.
+struct IoView {
+  const int64_t *__restrict__ io_ptrs;
+  const char *__restrict__ arg_base;
+  const int64_t *__restrict__ arg_offsets;
+  int batch;
+
+  __device__ __forceinline__ const int *offsets(int f) const {
+    if (io_ptrs) return global_ptr<int>(io_ptrs[2 * f + 1]);
+    return global_ptr<int>(reinterpret_cast<int64_t>(arg_base) + arg_offsets[f]);
+  }
+  __device__ __forceinline__ const int *indices(int f) const {
+    if (io_ptrs) return global_ptr<int>(io_ptrs[2 * f]);
+    return global_ptr<int>(reinterpret_cast<int64_t>(arg_base) + arg_offsets[f] +
+                           alignmem((static_cast<int64_t>(batch) + 1) * 4));
+  }
+};
+
+template <int F> struct BindingStorage {
+  int prefix[F + 1];      // prefix[f] = first global tile id of feature f
+  int bags_per_tile[F];
+};
+
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int t = __shfl_up(v, d, 64);
+    if (lane >= d) v += t;
+  }
+  return v;
+}
+
+// lookup_bytes[f]: bytes fetched per lookup (row + index); bag_bytes[f]: bytes per bag that do
+// not depend on its length (output row slice + offset); gran[f]: bags a workgroup of this
+// feature's schedule handles per pass (tiles are whole multiples of it).
+// fixed_tiles: if non-null, the tile count per feature is taken from it instead of from the
+// live offsets (static thread binding, for the ablation).
+// Returns the total number of tiles.  Ends with a barrier.
+template <int F, int BT>
+__device__ __forceinline__ int
+bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
+           const int *__restrict__ lookup_bytes, const int *__restrict__ bag_bytes,
+           const int *__restrict__ gran, const int *__restrict__ fixed_tiles) {
+  const int tid = threadIdx.x;
+  const int B = io.batch;
+  for (int f = tid; f < F; f += BT) {
+    const int g = gran[f];
+    const int max_tiles = (B + g - 1) / g;
+    int64_t want;
+    if (fixed_tiles) {
+      want = fixed_tiles[f];
+    } else {
+      const int *offs = io.offsets(f);
+      const int64_t lookups = static_cast<int64_t>(offs[B]) - offs[0];
+      const int64_t cost = lookups * lookup_bytes[f] + static_cast<int64_t>(B) * bag_bytes[f];
+      want = (cost + tile_bytes - 1) / tile_bytes;
+    }
+    int tiles = want < 1 ? 1 : (want > max_tiles ? max_tiles : static_cast<int>(want));
+    int bpt = 0;
+    if (B > 0) {
+      bpt = ((B + tiles - 1) / tiles + g - 1) / g * g;
+      tiles = (B + bpt - 1) / bpt;
+    } else {
+      tiles = 0;
+    }
+    s.bags_per_tile[f] = bpt;
+    s.prefix[f + 1] = tiles;
+  }
+  if (tid == 0) s.prefix[0] = 0;
+  __syncthreads();
+  if (tid < 64) {
+    int carry = 0;
+    for (int c = 0; c < F; c += 64) {
+      const int i = c + tid;
+      int v = i < F ? s.prefix[i + 1] : 0;
+      v = wave_inclusive_scan(v, tid) + carry;
+      if (i < F) s.prefix[i + 1] = v;
+      carry = __shfl(v, 63, 64);
+    }
+  }
+  __syncthreads();
+  return s.prefix[F];
+}
+
+// feature owning global tile id `tile` (0 <= tile < prefix[F]): largest f with prefix[f] <= tile
+template <int F>
+__device__ __forceinline__ int find_feature(const BindingStorage<F> &s, const int tile) {
+  int lo = 0, hi = F;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (s.prefix[mid] <= tile) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+} // namespace rfx

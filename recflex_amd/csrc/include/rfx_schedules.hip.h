@@ -1,0 +1,300 @@
+// The per-feature schedule bodies of the fused embedding kernel, written for 64-lane
+// wavefronts: every bag (one sample's lookups of one feature) is summed by a "team" of
+// T = X*Y lanes.  X lanes split the row into 16-byte vectors (column lanes), Y lanes split the
+// bag's lookups (lookup lanes) and are combined by a DPP / ds_swizzle / permlane butterfly.
+//
+//   T == 1          thread-per-bag          (team_bags)
+//   1 < T < 64      sub-wavefront-per-bag   (team_bags)
+//   T == 64         wavefront-per-bag       (team_bags)
+//   T == BT (256)   block-per-bag           (block_bags: indices staged in LDS, partial sums
+//                                            of the 4 wavefronts combined through LDS)
+//
+// Reference counterparts: ws::SparseSegmentReduce
+// (examples/csrc/include/warp_per_sample_kernel.cuh:10-82), obms::SparseSegmentReduce
+// (examples/csrc/include/one_block_multi_sample_kernel.cuh:9-126) and onehot::GatherSegments
+// (examples/csrc/include/onehot_kernel.cuh:14-87).  Semantics kept: sum pooling, empty bag ->
+// zeros, output row-major [batch, EMBED_DIM_SUM] with this feature at column embed_dim_offset.
+// Differences: 64-bit row addressing, tables may be fp32 / fp16 / int8 row-wise, the work unit
+// is a range of bags [bag_begin, bag_end) chosen at run time, and U lookups x UB bags x VPP
+// vectors are kept in flight per lane.
+#pragma once
+#include "rfx_crosslane.hip.h"
+#include "rfx_rows.hip.h"
+
+namespace rfx {
+
+// ---------------------------------------------------------------------------------------------
+// team_bags: teams of T <= 64 lanes; a workgroup of BT threads holds BT/T teams; team t sums
+// bags bag_begin + (t + k*TEAMS)*UB + [0, UB).
+//   U   lookups of one bag in flight per lookup lane
+//   UB  bags in flight per team (for short bags)
+//   VPP row vectors per lane per pass (a lane owns ceil(V/X) vectors; if that exceeds VPP the
+//       bag's index list is walked again for the next VPP vectors)
+// ---------------------------------------------------------------------------------------------
+template <int BT, int DT, int D, int X, int Y, int U, int UB, int VPP, int OVEC>
+__device__ __forceinline__ void
+team_bags(const char *__restrict__ table, const int *__restrict__ indices,
+          const int *__restrict__ offsets, float *__restrict__ out, const int esum,
+          const int col_off, const int bag_begin, const int bag_end) {
+  using R = Row<DT, D>;
+  constexpr int T = X * Y;
+  static_assert(T >= 1 && T <= 64 && (T & (T - 1)) == 0, "team must be a power of two <= 64");
+  static_assert(BT % T == 0 && BT % 64 == 0, "workgroup must hold whole teams");
+  constexpr int TEAMS = BT / T;
+  constexpr int VPL = ceil_div(R::V, X);
+  static_assert(VPP >= 1 && VPP <= VPL, "vectors per pass");
+  constexpr int VB = R::VB;
+  constexpr int EPV = R::EPV;
+
+  const int tid = threadIdx.x;
+  const int team = tid / T;
+  const int lt = tid - team * T;
+  const int y = lt / X;
+  const int x = lt - y * X;
+
+  for (int bag0 = bag_begin + team * UB; bag0 < bag_end; bag0 += TEAMS * UB) {
+    int beg[UB], end[UB];
+    {
+      int prev = offsets[bag0];
+#pragma unroll
+      for (int i = 0; i < UB; ++i) {
+        const int b = bag0 + i + 1;
+        const int next = offsets[b < bag_end ? b : bag_end];
+        beg[i] = prev;
+        end[i] = (bag0 + i < bag_end) ? next : prev;
+        prev = next;
+      }
+    }
+    int len_max = 0;
+#pragma unroll
+    for (int i = 0; i < UB; ++i) len_max = max(len_max, end[i] - beg[i]);
+
+#pragma unroll
+    for (int v0 = 0; v0 < VPL; v0 += VPP) {
+      float acc[UB][VPP][EPV];
+      float bias_acc[UB];
+#pragma unroll
+      for (int i = 0; i < UB; ++i) {
+        bias_acc[i] = 0.f;
+#pragma unroll
+        for (int v = 0; v < VPP; ++v)
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) acc[i][v][e] = 0.f;
+      }
+
+      // index of the lookup each (bag, unroll slot) will read next; -1 = none
+      int idx[UB][U];
+#pragma unroll
+      for (int i = 0; i < UB; ++i)
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int p = beg[i] + u * Y + y;
+          idx[i][u] = p < end[i] ? indices[p] : -1;
+        }
+
+      for (int base = 0; base < len_max; base += U * Y) {
+        Vec<VB> buf[UB][U][VPP];
+        f32x2 sb[UB][U];
+#pragma unroll
+        for (int i = 0; i < UB; ++i)
+#pragma unroll
+          for (int u = 0; u < U; ++u)
+            if (idx[i][u] >= 0) {
+              const char *row = table + static_cast<int64_t>(idx[i][u]) * R::STRIDE;
+#pragma unroll
+              for (int v = 0; v < VPP; ++v) {
+                const int c = x + (v0 + v) * X;
+                if (v0 + v < VPL && c < R::V) buf[i][u][v] = load_vec<VB>(row + c * VB);
+              }
+              if constexpr (DT == I8) sb[i][u] = load_scale_bias<D>(row);
+            }
+
+        // fetch the next round of indices while the rows are in flight
+        int nidx[UB][U];
+        const int nbase = base + U * Y;
+#pragma unroll
+        for (int i = 0; i < UB; ++i)
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            const int p = beg[i] + nbase + u * Y + y;
+            nidx[i][u] = p < end[i] ? indices[p] : -1;
+          }
+
+#pragma unroll
+        for (int i = 0; i < UB; ++i)
+#pragma unroll
+          for (int u = 0; u < U; ++u)
+            if (idx[i][u] >= 0) {
+#pragma unroll
+              for (int v = 0; v < VPP; ++v) {
+                const int c = x + (v0 + v) * X;
+                if (v0 + v < VPL && c < R::V)
+                  accumulate<DT, VB>(acc[i][v], buf[i][u][v], DT == I8 ? sb[i][u].x : 1.f);
+              }
+              if constexpr (DT == I8) bias_acc[i] += sb[i][u].y;
+            }
+
+#pragma unroll
+        for (int i = 0; i < UB; ++i)
+#pragma unroll
+          for (int u = 0; u < U; ++u) idx[i][u] = nidx[i][u];
+      }
+
+      if constexpr (Y > 1) {
+#pragma unroll
+        for (int i = 0; i < UB; ++i) {
+          if constexpr (DT == I8) bias_acc[i] = reduce_over_y<X, T>(bias_acc[i]);
+#pragma unroll
+          for (int v = 0; v < VPP; ++v)
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) acc[i][v][e] = reduce_over_y<X, T>(acc[i][v][e]);
+        }
+      }
+
+      if (y == 0) {
+#pragma unroll
+        for (int i = 0; i < UB; ++i) {
+          const int bag = bag0 + i;
+          if (bag < bag_end) {
+            float *dst = out + static_cast<int64_t>(bag) * esum + col_off;
+#pragma unroll
+            for (int v = 0; v < VPP; ++v) {
+              const int c = x + (v0 + v) * X;
+              if (v0 + v < VPL && c < R::V) {
+                if constexpr (DT == I8) {
+#pragma unroll
+                  for (int e = 0; e < EPV; ++e) acc[i][v][e] += bias_acc[i];
+                }
+                store_floats<EPV, OVEC>(dst + c * EPV, acc[i][v]);
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// block_bags: the whole workgroup sums one bag at a time (long bags).  The bag's indices are
+// staged in LDS in chunks of CHUNK with coalesced loads; lane (y, x) reads index y + k*Y of the
+// chunk and vector(s) x of the row; the Y lookup lanes inside a wavefront are combined with the
+// cross-lane butterfly, the BT/64 wavefronts through LDS, and the result is written with
+// coalesced 4-byte stores.
+// ---------------------------------------------------------------------------------------------
+template <int BT, int DT, int D, int X, int CHUNK> struct BlockBagStorage {
+  using R = Row<DT, D>;
+  static constexpr int VPL = ceil_div(R::V, X);
+  static constexpr int COLS = X * VPL * R::EPV; // >= D
+  int idx[CHUNK];
+  float part[BT / 64][COLS];
+  float part_bias[BT / 64];
+};
+
+template <int BT, int DT, int D, int X, int U, int CHUNK>
+__device__ __forceinline__ void
+block_bags(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ table,
+           const int *__restrict__ indices, const int *__restrict__ offsets,
+           float *__restrict__ out, const int esum, const int col_off, const int bag_begin,
+           const int bag_end) {
+  using R = Row<DT, D>;
+  static_assert(X >= 1 && X <= 64 && (X & (X - 1)) == 0, "column lanes");
+  static_assert(BT % 64 == 0 && CHUNK % BT == 0, "chunk must be whole workgroup loads");
+  constexpr int Y = BT / X;
+  constexpr int WAVES = BT / 64;
+  constexpr int VPL = ceil_div(R::V, X);
+  constexpr int VB = R::VB;
+  constexpr int EPV = R::EPV;
+  constexpr int COLS = X * VPL * EPV;
+
+  const int tid = threadIdx.x;
+  const int y = tid / X;
+  const int x = tid - y * X;
+  const int wave = tid / 64;
+  const int lane = tid - wave * 64;
+
+  for (int bag = bag_begin; bag < bag_end; ++bag) {
+    const int beg = offsets[bag];
+    const int end = offsets[bag + 1];
+
+    float acc[VPL][EPV];
+    float bias_acc = 0.f;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v)
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) acc[v][e] = 0.f;
+
+    // also orders the previous bag's reads of s.part / s.idx before this bag's writes
+    __syncthreads();
+    for (int c0 = beg; c0 < end; c0 += CHUNK) {
+      const int n = min(CHUNK, end - c0);
+      if (c0 != beg) __syncthreads();
+#pragma unroll
+      for (int i = 0; i < CHUNK; i += BT)
+        if (i + tid < n) s.idx[i + tid] = indices[c0 + i + tid];
+      __syncthreads();
+
+      for (int base = 0; base < n; base += U * Y) {
+        Vec<VB> buf[U][VPL];
+        f32x2 sb[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int p = base + u * Y + y;
+          ok[u] = p < n;
+          if (ok[u]) {
+            const char *row = table + static_cast<int64_t>(s.idx[p]) * R::STRIDE;
+#pragma unroll
+            for (int v = 0; v < VPL; ++v) {
+              const int c = x + v * X;
+              if (c < R::V) buf[u][v] = load_vec<VB>(row + c * VB);
+            }
+            if constexpr (DT == I8) sb[u] = load_scale_bias<D>(row);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (ok[u]) {
+#pragma unroll
+            for (int v = 0; v < VPL; ++v) {
+              const int c = x + v * X;
+              if (c < R::V) accumulate<DT, VB>(acc[v], buf[u][v], DT == I8 ? sb[u].x : 1.f);
+            }
+            if constexpr (DT == I8) bias_acc += sb[u].y;
+          }
+      }
+    }
+
+    // combine the lookup lanes that share a wavefront
+    if constexpr (X < 64) {
+      if constexpr (DT == I8) bias_acc = reduce_over_y<X, 64>(bias_acc);
+#pragma unroll
+      for (int v = 0; v < VPL; ++v)
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) acc[v][e] = reduce_over_y<X, 64>(acc[v][e]);
+    }
+    if (lane < X) {
+#pragma unroll
+      for (int v = 0; v < VPL; ++v)
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) s.part[wave][(x + v * X) * EPV + e] = acc[v][e];
+      if (lane == 0) s.part_bias[wave] = bias_acc;
+    }
+    __syncthreads();
+
+    float *dst = out + static_cast<int64_t>(bag) * esum + col_off;
+    for (int j = tid; j < D; j += BT) {
+      float t = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) t += s.part[w][j];
+      if constexpr (DT == I8) {
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) t += s.part_bias[w];
+      }
+      dst[j] = t;
+    }
+  }
+  (void)COLS;
+}
+
+} // namespace rfx

@@ -1,0 +1,116 @@
+"""ctypes bindings of a generated ``librecom.so`` (``recom_*`` in ``include/recflex_hip.h``).
+
+Stands where the reference calls ``torch.ops.load_library(librecom_path)`` and
+``torch.ops.recom.{process,get_max_concurrent_blocks,get_gpu_pointers_array}``
+(``RecFlex/rec_modules.py:71-72,82-94``).  Each ``RecomLib`` owns its own ``dlopen`` handle, so
+any number of emitted kernels can be used in one process.
+"""
+
+import ctypes
+import os
+from typing import List, Optional
+
+_I32P = ctypes.POINTER(ctypes.c_int32)
+
+
+class RecomInfo(ctypes.Structure):
+    _fields_ = [
+        ("abi_version", ctypes.c_int32),
+        ("num_features", ctypes.c_int32),
+        ("embed_dim_sum", ctypes.c_int32),
+        ("block_threads", ctypes.c_int32),
+        ("occupancy", ctypes.c_int32),
+        ("num_bodies", ctypes.c_int32),
+        ("timing", ctypes.c_int32),
+        ("tile_bytes", ctypes.c_int32),
+        ("static_binding", ctypes.c_int32),
+        ("reserved", ctypes.c_int32 * 7),
+    ]
+
+
+class RecomProcessArgs(ctypes.Structure):
+    _fields_ = [
+        ("d_embed_table_ptrs", ctypes.c_void_p),
+        ("d_io_ptrs", ctypes.c_void_p),
+        ("d_arg_buffers", ctypes.c_void_p),
+        ("d_arg_buffer_offsets", ctypes.c_void_p),
+        ("d_output", ctypes.c_void_p),
+        ("batch", ctypes.c_int32),
+        ("tile_bytes", ctypes.c_int32),
+        ("grid_blocks", ctypes.c_int32),
+        ("d_times", ctypes.c_void_p),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+RECOM_ABI_VERSION = 1
+EXPORTED_SYMBOLS = ("recom_get_info", "recom_get_feature_tables",
+                    "recom_get_max_concurrent_blocks", "recom_process")
+
+
+class RecomError(RuntimeError):
+    def __init__(self, func: str, code: int):
+        super().__init__(f"{func} failed with hipError_t {code}")
+        self.code = code
+
+
+class RecomLib:
+    def __init__(self, path: str):
+        if not os.path.exists(path):
+            raise FileNotFoundError(f"{path} does not exist; build it first (the HIP library is "
+                                    "required, there is no fallback path)")
+        self.path = os.path.abspath(path)
+        self.lib = ctypes.CDLL(self.path)
+        for name in EXPORTED_SYMBOLS:
+            if not hasattr(self.lib, name):
+                raise RecomError(f"{path}: missing symbol {name}", -1)
+        self.lib.recom_get_info.restype = ctypes.c_int
+        self.lib.recom_get_info.argtypes = [ctypes.POINTER(RecomInfo)]
+        self.lib.recom_get_feature_tables.restype = ctypes.c_int
+        self.lib.recom_get_feature_tables.argtypes = [_I32P, _I32P, _I32P, _I32P]
+        self.lib.recom_get_max_concurrent_blocks.restype = ctypes.c_int
+        self.lib.recom_get_max_concurrent_blocks.argtypes = [_I32P]
+        self.lib.recom_process.restype = ctypes.c_int
+        self.lib.recom_process.argtypes = [ctypes.POINTER(RecomProcessArgs)]
+
+        self.info = RecomInfo()
+        rc = self.lib.recom_get_info(ctypes.byref(self.info))
+        if rc != 0:
+            raise RecomError("recom_get_info", rc)
+        if self.info.abi_version != RECOM_ABI_VERSION:
+            raise RecomError(f"{path}: ABI version {self.info.abi_version} != {RECOM_ABI_VERSION}", -1)
+        f = self.info.num_features
+        arrs = [(ctypes.c_int32 * f)() for _ in range(4)]
+        rc = self.lib.recom_get_feature_tables(*arrs)
+        if rc != 0:
+            raise RecomError("recom_get_feature_tables", rc)
+        self.embed_dims: List[int] = list(arrs[0])
+        self.embed_dim_offsets: List[int] = list(arrs[1])
+        self.dtypes: List[int] = list(arrs[2])
+        self.row_strides: List[int] = list(arrs[3])
+
+    @property
+    def num_features(self) -> int:
+        return self.info.num_features
+
+    @property
+    def embed_dim_sum(self) -> int:
+        return self.info.embed_dim_sum
+
+    def get_max_concurrent_blocks(self) -> int:
+        out = ctypes.c_int32(0)
+        rc = self.lib.recom_get_max_concurrent_blocks(ctypes.byref(out))
+        if rc != 0:
+            raise RecomError("recom_get_max_concurrent_blocks", rc)
+        return out.value
+
+    def process(self, table_ptrs: int, output: int, batch: int, *, io_ptrs: int = 0,
+                arg_buffers: int = 0, arg_buffer_offsets: int = 0, tile_bytes: int = 0,
+                grid_blocks: int = 0, times: int = 0, stream: int = 0) -> None:
+        """All pointer arguments are raw device addresses (``tensor.data_ptr()``)."""
+        args = RecomProcessArgs(table_ptrs or None, io_ptrs or None, arg_buffers or None,
+                                arg_buffer_offsets or None, output or None, batch, tile_bytes,
+                                grid_blocks, times or None, stream or None)
+        rc = self.lib.recom_process(ctypes.byref(args))
+        if rc != 0:
+            raise RecomError("recom_process", rc)

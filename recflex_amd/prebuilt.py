@@ -1,0 +1,152 @@
+"""Named, reproducible models (workload + per-feature schedules) whose fused-kernel libraries
+are built ahead of time, in-tree, under ``recflex_amd/_models/<name>/build/``.
+
+GPU machines only load what is already built here; ``ensure_built`` compiles a model only if
+its library is missing.  Names:
+
+``c1`` .. ``c5``     the five benchmark configurations at full size, default (untuned) schedules
+``c3_tuned``       C3 with the schedules in ``recflex_amd/tuned/c3_schedule.json`` if present
+``c2s`` .. ``c5s``   shrunken C2..C5 (fewer rows / features / samples) that a CPU checker can follow
+``variants``       one feature per (element type, dim, schedule candidate) over a spread of the
+                   candidate space of all four templates, with ragged bags (up to ~1500 lookups)
+                   and integer-valued tables, so that sums are exact in any order
+``edge``           dims that force 8- and 4-byte row vectors and unaligned output columns
+"""
+
+import json
+import os
+from typing import Callable, Dict, List, NamedTuple, Optional, Tuple
+
+import numpy as np
+
+from .code_emitter import MetaData
+from .model_build import FeatSchedules, build_model, default_feat_schedules, load_feat_schedules
+from .schedules import (BlockPerBagSchedule, SubWavefrontPerBagSchedule, ThreadPerBagSchedule,
+                        WavefrontPerBagSchedule)
+from .workloads import FeatureSpec, Workload, make_workload
+
+PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
+MODELS_DIR = os.path.join(PACKAGE_DIR, "_models")
+TUNED_DIR = os.path.join(PACKAGE_DIR, "tuned")
+BLOCK_THREADS = 256
+
+
+class ModelSpec(NamedTuple):
+    workload: Workload
+    feat_schedules: FeatSchedules
+    occupancy: Optional[int]
+
+
+def metas_of(wl: Workload) -> List[MetaData]:
+    return [MetaData(f.dim, f.data_type) for f in wl.features]
+
+
+def expected_bag_len(f: FeatureSpec) -> float:
+    return f.mean_bag * (1.0 - f.empty_frac)
+
+
+def _default(wl: Workload, occupancy: Optional[int] = None) -> ModelSpec:
+    fs = default_feat_schedules(metas_of(wl), [expected_bag_len(f) for f in wl.features], BLOCK_THREADS)
+    return ModelSpec(wl, fs, occupancy)
+
+
+def _tuned(wl: Workload, fname: str) -> ModelSpec:
+    path = os.path.join(TUNED_DIR, fname)
+    if not os.path.exists(path):
+        return _default(wl)
+    with open(path) as f:
+        doc = json.load(f)
+    entries = doc["schedules"] if isinstance(doc, dict) else doc
+    occupancy = doc.get("occupancy") if isinstance(doc, dict) else None
+    tmp = os.path.join(MODELS_DIR, f".{fname}.entries.json")
+    os.makedirs(MODELS_DIR, exist_ok=True)
+    with open(tmp, "w") as f:
+        json.dump(entries, f)
+    fs = load_feat_schedules(tmp, BLOCK_THREADS)
+    os.remove(tmp)
+    assert len(fs) == wl.num_features
+    return ModelSpec(wl, fs, occupancy)
+
+
+def _variants() -> ModelSpec:
+    """A spread of every template's candidate list for each (element type, dim)."""
+    rng = np.random.default_rng(77)
+    feats: List[FeatureSpec] = []
+    scheds: FeatSchedules = []
+    combos = [("float", 8), ("float", 32), ("float", 128), ("float", 256),
+              ("half", 16), ("half", 64), ("half", 256),
+              ("int8", 16), ("int8", 64), ("int8", 128)]
+    for data_type, dim in combos:
+        meta = MetaData(dim, data_type)
+        for cls, take in ((ThreadPerBagSchedule, 3), (SubWavefrontPerBagSchedule, 8),
+                          (WavefrontPerBagSchedule, 4), (BlockPerBagSchedule, 2)):
+            sched = cls(meta, BLOCK_THREADS)
+            cands = sched.GenParamCandidates()
+            if not cands:
+                continue
+            picks = sorted(set(int(i) for i in np.linspace(0, len(cands) - 1, min(take, len(cands)))))
+            for i in picks:
+                mean = float(rng.choice([0.7, 3.0, 17.0, 90.0]))
+                if cls is BlockPerBagSchedule:
+                    mean = float(rng.choice([40.0, 1500.0]))     # > one LDS chunk of indices
+                feats.append(FeatureSpec(int(rng.integers(50, 5000)), dim, data_type, mean, False,
+                                         0.1, 1.0))
+                scheds.append((sched, cands[i]))
+    return ModelSpec(Workload("variants", 96, 4242, tuple(feats), "integer"), scheds, None)
+
+
+def _edge() -> ModelSpec:
+    dims = [("float", 1), ("float", 2), ("float", 6), ("float", 12), ("float", 20), ("half", 2),
+            ("half", 4), ("half", 12), ("int8", 4), ("int8", 8), ("int8", 24), ("float", 3)]
+    feats = [FeatureSpec(300 + 7 * i, d, t, 5.0, False, 0.2, 0.9) for i, (t, d) in enumerate(dims)]
+    wl = Workload("edge", 70, 99, tuple(feats), "integer")
+    fs = default_feat_schedules(metas_of(wl), [4.0] * len(feats), BLOCK_THREADS)
+    return ModelSpec(wl, fs, None)
+
+
+_SPECS: Dict[str, Callable[[], ModelSpec]] = {
+    "c1": lambda: _default(make_workload("C1")),
+    "c2": lambda: _default(make_workload("C2")),
+    "c3": lambda: _default(make_workload("C3")),
+    "c4": lambda: _default(make_workload("C4")),
+    "c5": lambda: _default(make_workload("C5")),
+    "c3_tuned": lambda: _tuned(make_workload("C3"), "c3_schedule.json"),
+    "c2s": lambda: _default(make_workload("C2", batch=512, max_rows=200_000)),
+    "c3s": lambda: _default(make_workload("C3", batch=192, max_rows=60_000)),
+    "c4s": lambda: _default(make_workload("C4", batch=128, num_features=48, max_rows=30_000)),
+    "c5s": lambda: _default(make_workload("C5", batch=256, num_features=24, max_rows=50_000)),
+    "variants": _variants,
+    "edge": _edge,
+}
+
+
+def model_names() -> List[str]:
+    return list(_SPECS)
+
+
+def model_spec(name: str) -> ModelSpec:
+    if name not in _SPECS:
+        raise KeyError(f"unknown prebuilt model {name!r}; known: {model_names()}")
+    return _SPECS[name]()
+
+
+def model_dir(name: str) -> str:
+    return os.path.join(MODELS_DIR, name)
+
+
+def lib_path(name: str) -> str:
+    return os.path.join(model_dir(name), "build", "librecom.so")
+
+
+def build(name: str) -> str:
+    spec = model_spec(name)
+    return build_model(model_dir(name), spec.feat_schedules, rebuild=True, occupancy=spec.occupancy)
+
+
+def ensure_built(name: str) -> str:
+    path = lib_path(name)
+    return path if os.path.exists(path) else build(name)
+
+
+def build_all(names: Optional[List[str]] = None) -> Dict[str, str]:
+    return {name: build(name) for name in (names or model_names())}

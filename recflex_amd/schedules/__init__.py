@@ -1,0 +1,88 @@
+"""Schedule templates for the gfx950 fused embedding kernel.
+
+``SCHEDULE_MAPPING`` plays the role of ``globals()`` of the reference's ``examples/tune.py``
+(``tune.py:78`` passes it as ``schedule_mapping``): class name in ``schedule_config.txt`` ->
+schedule class.
+"""
+
+from typing import Dict, NamedTuple, Tuple, Type
+
+from recflex_amd.code_emitter.schedule_base import ScheduleBase, MetaData
+from .team import (TeamParams, TeamScheduleBase, ThreadPerBagSchedule, ThreadPerBagParams,
+                   SubWavefrontPerBagSchedule, SubWavefrontPerBagParams,
+                   WavefrontPerBagSchedule, WavefrontPerBagParams, next_pow2)
+from .block_per_bag import BlockPerBagSchedule, BlockPerBagParams
+from .reference_names import (OneHotSchedule, OneHotMultiBlockSchedule, WarpPerSampleSchedule,
+                              OneBlockMultiSampleSchedule, MultiBlockPerSampleSchedule,
+                              ReduceByKeySchedule, OneHotParams, OneHotMultiBlockParams,
+                              WarpPerSampleParams, OneBlockMultiSampleParams,
+                              MultiBlockPerSampleParams, ReduceByKeyParams)
+
+SCHEDULE_MAPPING: Dict[str, Type[ScheduleBase]] = {
+    cls.__name__: cls
+    for cls in (ThreadPerBagSchedule, SubWavefrontPerBagSchedule, WavefrontPerBagSchedule,
+                BlockPerBagSchedule, OneHotSchedule, OneHotMultiBlockSchedule,
+                WarpPerSampleSchedule, OneBlockMultiSampleSchedule,
+                MultiBlockPerSampleSchedule, ReduceByKeySchedule)
+}
+
+PARAM_TYPES: Dict[str, Type[NamedTuple]] = {
+    "ThreadPerBagSchedule": ThreadPerBagParams,
+    "SubWavefrontPerBagSchedule": SubWavefrontPerBagParams,
+    "WavefrontPerBagSchedule": WavefrontPerBagParams,
+    "BlockPerBagSchedule": BlockPerBagParams,
+    "OneHotSchedule": TeamParams,
+    "OneHotMultiBlockSchedule": TeamParams,
+    "WarpPerSampleSchedule": TeamParams,
+    "OneBlockMultiSampleSchedule": TeamParams,
+    "MultiBlockPerSampleSchedule": BlockPerBagParams,
+    "ReduceByKeySchedule": BlockPerBagParams,
+}
+
+
+def default_schedule(meta: MetaData, mean_bag_len: float = 1.0,
+                     block_threads: int = 256) -> Tuple[ScheduleBase, NamedTuple]:
+    """Untuned starting point for one feature from its row size and mean bag length: enough
+    column lanes that a lane owns one or two 16-byte vectors, lookup lanes only for long bags,
+    and four to eight independent row loads in flight per lane."""
+    v = meta.row_vectors
+    x = min(64, next_pow2(v))
+    if v > 1 and x * meta.vec_bytes >= 256 and mean_bag_len < 8:
+        x //= 2                      # short bags of wide rows: two vectors per lane
+    vpl = -(-v // x)
+    if mean_bag_len <= 1.5:
+        bags = 4 if vpl == 1 else 2
+        team = x
+        if team == 1:
+            return ThreadPerBagSchedule(meta, block_threads), ThreadPerBagParams(1, bags, vpl)
+        if team == 64:
+            return WavefrontPerBagSchedule(meta, block_threads), WavefrontPerBagParams(64, 1, vpl)
+        return (SubWavefrontPerBagSchedule(meta, block_threads),
+                SubWavefrontPerBagParams(x, 1, 1, bags, vpl))
+    items = 4 if vpl <= 2 else 2
+    if mean_bag_len < 24:
+        y = 1
+    elif mean_bag_len < 96:
+        y = max(1, min(4, 64 // x))
+    else:
+        y = max(1, 64 // x)
+    if mean_bag_len >= 512 and x >= 16:
+        return (BlockPerBagSchedule(meta, block_threads),
+                BlockPerBagParams(min(x, 64), items, 4 * block_threads))
+    team = x * y
+    if team == 1:
+        return ThreadPerBagSchedule(meta, block_threads), ThreadPerBagParams(items, 1, vpl)
+    if team == 64:
+        return WavefrontPerBagSchedule(meta, block_threads), WavefrontPerBagParams(x, items, vpl)
+    return (SubWavefrontPerBagSchedule(meta, block_threads),
+            SubWavefrontPerBagParams(x, y, items, 1, vpl))
+
+
+def schedule_from_config(entry: dict, meta: MetaData, block_threads: int = 256
+                         ) -> Tuple[ScheduleBase, NamedTuple]:
+    """Inverse of ``CodeEmitter.serialize_config`` for one feature:
+    ``{"schedule": ClassName, "params": {...}}`` -> (schedule object, params tuple)."""
+    name = entry["schedule"]
+    if name not in SCHEDULE_MAPPING:
+        raise KeyError(f"unknown schedule class {name!r}")
+    return SCHEDULE_MAPPING[name](meta, block_threads), PARAM_TYPES[name](**entry["params"])

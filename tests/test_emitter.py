@@ -1,0 +1,164 @@
+"""Code emitter and schedule templates (host logic only: what is emitted, not how it runs)."""
+
+import json
+import os
+import re
+
+import pytest
+
+from recflex_amd.code_emitter import CodeEmitter, MetaData, ScheduleBase, InputStats
+from recflex_amd.schedules import (SCHEDULE_MAPPING, BlockPerBagParams, BlockPerBagSchedule,
+                                   SubWavefrontPerBagParams, SubWavefrontPerBagSchedule,
+                                   ThreadPerBagSchedule, WavefrontPerBagParams,
+                                   WavefrontPerBagSchedule, default_schedule, schedule_from_config)
+from recflex_amd.schedules.team import TeamParams, fits_registers
+
+
+def test_metadata_row_formats():
+    m = MetaData(64)
+    assert (m.data_type, m.row_stride, m.row_bytes, m.vec_bytes, m.row_vectors, m.elems_per_vector) == \
+        ("float", 256, 256, 16, 16, 4)
+    m = MetaData(128, "half")
+    assert (m.row_stride, m.row_bytes, m.vec_bytes, m.row_vectors, m.elems_per_vector) == (256, 256, 16, 16, 8)
+    m = MetaData(128, "int8")
+    assert (m.row_stride, m.row_bytes, m.vec_bytes, m.row_vectors, m.elems_per_vector) == (144, 132, 16, 8, 16)
+    m = MetaData(6)
+    assert (m.vec_bytes, m.row_vectors) == (8, 3)
+    with pytest.raises(ValueError):
+        MetaData(3, "int8").vec_bytes
+    with pytest.raises(ValueError):
+        MetaData(8, "bfloat16").dtype_id
+
+
+def test_reference_schedule_names_resolve():
+    """The class names used by the reference's schedule_config.txt files."""
+    for name in ("OneHotSchedule", "OneHotMultiBlockSchedule", "WarpPerSampleSchedule",
+                 "OneBlockMultiSampleSchedule", "MultiBlockPerSampleSchedule", "ReduceByKeySchedule",
+                 "ThreadPerBagSchedule", "SubWavefrontPerBagSchedule", "WavefrontPerBagSchedule",
+                 "BlockPerBagSchedule"):
+        cls = SCHEDULE_MAPPING[name]
+        assert issubclass(cls, ScheduleBase)
+        cands = cls(MetaData(16), 256).GenParamCandidates()
+        assert len(cands) > 0
+        assert len(set(cands)) == len(cands)
+
+
+@pytest.mark.parametrize("dt,dim", [("float", 8), ("float", 128), ("half", 16), ("half", 256),
+                                    ("int8", 128), ("float", 12)])
+def test_candidates_are_valid_and_emit(dt, dim):
+    meta = MetaData(dim, dt)
+    total = 0
+    for cls in (ThreadPerBagSchedule, SubWavefrontPerBagSchedule, WavefrontPerBagSchedule, BlockPerBagSchedule):
+        sched = cls(meta, 256)
+        for p in sched.GenParamCandidates():
+            body = sched.EmitScheduleBody(p)          # raises on invalid parameters
+            assert "rfx::" in body
+            g = sched.TileGranularity(p)
+            assert g >= 1 and 256 % g == 0 or g % 256 == 0 or g > 0
+            if cls is not BlockPerBagSchedule:
+                tp = sched.team_params(p)
+                assert fits_registers(meta, tp)
+                assert tp.lanes_x * tp.lanes_y <= 64
+            total += 1
+    assert 4 <= total <= 200
+
+
+def test_invalid_params_rejected():
+    meta = MetaData(64)
+    with pytest.raises(ValueError):
+        SubWavefrontPerBagSchedule(meta, 256).EmitScheduleBody(SubWavefrontPerBagParams(3, 1, 1, 1, 1))
+    with pytest.raises(ValueError):
+        SubWavefrontPerBagSchedule(meta, 256).EmitScheduleBody(SubWavefrontPerBagParams(16, 8, 1, 1, 1))
+    with pytest.raises(ValueError):
+        WavefrontPerBagSchedule(meta, 256).EmitScheduleBody(WavefrontPerBagParams(16, 1, 5))
+    with pytest.raises(ValueError):
+        BlockPerBagSchedule(meta, 256).EmitScheduleBody(BlockPerBagParams(16, 1, 1000))
+
+
+def _emitter(dims_types, sched_fn=None):
+    fs = []
+    for d, t, pf in dims_types:
+        fs.append(default_schedule(MetaData(d, t), pf, 256))
+    return CodeEmitter(fs)
+
+
+def test_body_dedup_and_tables():
+    """Identical (LDS type, body) pairs are emitted once (codegen.py:233-243)."""
+    em = _emitter([(32, "float", 4), (32, "float", 4), (64, "float", 4), (32, "float", 4), (32, "half", 4)])
+    id_map, bodies = em.dedup()
+    assert id_map == {0: 0, 1: 0, 2: 2, 3: 0, 4: 4} and bodies == [0, 2, 4]
+    src = em.emit_kernel(occupancy=4)
+    assert len(re.findall(r"void ProcessFeat\d+\(", src)) == 3
+    assert "constexpr int NUM_FEATS = 5;" in src and "constexpr int EMBED_DIM_SUM = 192;" in src
+    assert "__launch_bounds__(BLOCK_THREADS, 4)" in src
+    m = re.search(r"c_embed_dim_offsets\[\] = \{\s*([\d,\s]+)\}", src)
+    assert [int(v) for v in m.group(1).split(",")] == [0, 32, 64, 128, 160, 192]
+    m = re.search(r"c_process_func_ids\[\] = \{\s*([\d,\s]+)\}", src)
+    assert [int(v) for v in m.group(1).split(",")] == [0, 0, 2, 0, 4]
+    # bytes per lookup = row bytes + int32 index; per bag = fp32 output slice + one offset
+    m = re.search(r"c_lookup_bytes\[\] = \{\s*([\d,\s]+)\}", src)
+    assert [int(v) for v in m.group(1).split(",")] == [132, 132, 260, 132, 68]
+    m = re.search(r"c_bag_bytes\[\] = \{\s*([\d,\s]+)\}", src)
+    assert [int(v) for v in m.group(1).split(",")] == [132, 132, 260, 132, 132]
+
+
+def test_output_vector_width_follows_column_alignment():
+    assert _emitter([(32, "float", 4), (64, "float", 4)]).out_vec() == 4
+    assert _emitter([(6, "float", 4), (64, "float", 4)]).out_vec() == 2
+    assert _emitter([(3, "float", 4), (64, "float", 4)]).out_vec() == 1
+
+
+def test_emit_variants_and_file_update(tmp_path):
+    em = _emitter([(32, "float", 4), (128, "int8", 50)])
+    f = tmp_path / "process.hip"
+    em.emit(str(f), occupancy=2, timing=True)
+    src = f.read_text()
+    assert "TIMING = true" in src and "s_memtime" in src and "atomicAdd(&d_times[feat_idx]" in src
+    assert 'extern "C" int recom_process' in src and 'extern "C" int recom_get_info' in src
+    mtime = f.stat().st_mtime_ns
+    em.emit(str(f), occupancy=2, timing=True)            # unchanged -> not rewritten
+    assert f.stat().st_mtime_ns == mtime
+    em.emit(str(f), occupancy=2, timing=False, fixed_task_block_nums=[3, 9])
+    src = f.read_text()
+    assert "STATIC_BINDING = true" in src and "c_fixed_task_block_nums" in src
+    em.emit(str(f), inline=False)
+    assert "__noinline__ void ProcessFeat0" in f.read_text()
+    h = tmp_path / "preprocess.cpp"
+    em.emit_host(str(h))
+    hsrc = h.read_text()
+    assert "recom_host_preprocess_feat" in hsrc and hsrc.count("static int PreprocFeat") == 1
+    c = tmp_path / "CMakeLists.txt"
+    em.emit_cmake_list(str(c), code_fname="process.hip", host_fname="preprocess.cpp")
+    csrc = c.read_text()
+    assert "--offload-arch=gfx950" in csrc and "-packed-fp32-ops" in csrc and "librecom.so" in csrc
+
+
+def test_serialize_round_trip(tmp_path):
+    em = _emitter([(32, "float", 1), (128, "half", 40), (128, "int8", 300), (256, "float", 900)])
+    cfg = em.serialize_config()
+    assert [c["schedule"] for c in cfg] == [type(s).__name__ for s, _ in em.feat_schedules]
+    p = tmp_path / "schedule.json"
+    em.dump_key(str(p))
+    back = json.loads(p.read_text())
+    for entry, (sched, params) in zip(back, em.feat_schedules):
+        s2, p2 = schedule_from_config(entry, sched.meta, 256)
+        assert type(s2) is type(sched) and p2 == params
+    from recflex_amd.model_build import load_feat_schedules
+    fs = load_feat_schedules(str(p))
+    assert [p for _, p in fs] == [p for _, p in em.feat_schedules]
+    assert [s.meta for s, _ in fs] == [s.meta for s, _ in em.feat_schedules]
+
+
+def test_default_schedule_covers_all_templates():
+    kinds = set()
+    for dt in ("float", "half", "int8"):
+        for dim in (8, 16, 32, 64, 128, 256):
+            for pf in (1, 4, 30, 120, 800):
+                if dt == "int8" and dim < 16:
+                    continue
+                s, p = default_schedule(MetaData(dim, dt), pf)
+                s.EmitScheduleBody(p)
+                kinds.add(type(s).__name__)
+    assert kinds == {"ThreadPerBagSchedule", "SubWavefrontPerBagSchedule", "WavefrontPerBagSchedule",
+                     "BlockPerBagSchedule"} or kinds >= {"SubWavefrontPerBagSchedule", "WavefrontPerBagSchedule",
+                                                         "BlockPerBagSchedule"}
