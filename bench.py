@@ -1,0 +1,266 @@
+"""Benchmark of the fused-embedding hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--also c1,c2,c5]
+
+A step is one launch of the fused kernel over one batch of the synthetic workload whose inputs
+(tables, indices, offsets) and output buffer are already resident in HBM.  Prints ONE JSON line:
+``value`` is the achieved algorithmic bandwidth in GB/s of the headline workload (C3, the
+heterogeneous 100-feature configuration), next to kernel microseconds, pooled lookups per second,
+the roofline object for ``FusedKnl`` and the CPU baseline (the oracle: per-feature torch
+``embedding_bag(mode="sum")`` + concat on the host cores) timed in the same run, which is also
+the correctness check of the GPU result.  ``--also`` adds the same figures for further
+configurations under ``"configs"``.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0   # MI355X, HBM3E, published
+METRIC = "fused-kernel us + achieved HBM GB/s (% of MI355X peak) per model config"
+
+TOL = {"float": (1e-5, 1e-6), "half": (1e-3, 1e-6), "int8": (1e-3, 1e-6)}
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=10)
+    p.add_argument("--workload", type=str, default="c3",
+                   help="headline configuration (prebuilt model name: c1..c5, c3_tuned)")
+    p.add_argument("--also", type=str, default="c1,c2,c5",
+                   help="comma-separated further configurations reported under 'configs'")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / check leg")
+    p.add_argument("--tile-bytes", type=int, default=0)
+    p.add_argument("--grid-blocks", type=int, default=0)
+    p.add_argument("--copy-calibration", type=int, default=0,
+                   help="also launch one plain device-to-device copy of this many bytes (for "
+                        "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    p.add_argument("--cpu-features", type=int, default=0,
+                   help="bound the CPU leg to this many features (0 = choose from the size)")
+    return p.parse_args()
+
+
+def pick_model(name: str) -> str:
+    """Prefer the tuned build of a configuration when its schedule file exists."""
+    from recflex_amd import prebuilt
+    tuned = f"{name}_tuned"
+    if tuned in prebuilt.model_names() and \
+            os.path.exists(os.path.join(prebuilt.TUNED_DIR, f"{name}_schedule.json")):
+        return tuned
+    return name
+
+
+def cpu_leg(wl, tables, indices, offsets, gpu_out, max_features: int):
+    """Times the oracle on the host cores over a bounded sample (the first ``n`` features that
+    keep the work near 10-30 s) and checks the GPU output of those features against it."""
+    import numpy as np
+    import torch
+    from oracle import oracle
+    from recflex_amd.workloads import row_bytes
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    cores = torch.get_num_threads()
+    lookups = [len(i) for i in indices]
+    # bound the sample: at most ~60 M lookups (a few seconds per pass on a server CPU)
+    budget, n, acc = 60_000_000, 0, 0
+    while n < wl.num_features and (n == 0 or acc + lookups[n] <= budget):
+        acc += lookups[n]
+        n += 1
+    if max_features:
+        n = min(n, max_features)
+    feats = list(range(n))
+    host_tables = []
+    for f in feats:
+        spec = wl.features[f]
+        host_tables.append(oracle.decode_table(tables[f].cpu().numpy(), spec.dim, spec.data_type))
+    idx = [indices[f] for f in feats]
+    off = [offsets[f] for f in feats]
+
+    want = oracle.pooled_sum_torch(host_tables, idx, off)            # warm-up + the check values
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < 5.0 and len(times) < 200):
+        t0 = time.perf_counter()
+        oracle.pooled_sum_torch(host_tables, idx, off)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[len(times) // 2]
+    sample_bytes = sum(lookups[f] * (row_bytes(wl.features[f].dim, wl.features[f].data_type) + 4)
+                       + (wl.batch + 1) * 4 + wl.batch * wl.features[f].dim * 4 for f in feats)
+
+    ok, worst = True, 0.0
+    col = 0
+    got = gpu_out[:, :sum(wl.features[f].dim for f in feats)].cpu().numpy()
+    for f in feats:
+        spec = wl.features[f]
+        rtol, atol = TOL[spec.data_type]
+        good, max_abs, max_rel = oracle.within_tolerance(got[:, col:col + spec.dim],
+                                                         want[:, col:col + spec.dim], rtol, atol)
+        ok = ok and good
+        worst = max(worst, max_rel)
+        col += spec.dim
+    return {
+        "value": sample_bytes / t / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": f"features 0..{n - 1} of {wl.num_features} at full batch {wl.batch} "
+                  f"({sum(lookups[f] for f in feats)} lookups), median of {len(times)} passes of per-feature "
+                  f"torch embedding_bag(sum)+cat on fp32 host tables"
+                  + (" (fp16/int8 tables dequantised to fp32 beforehand, untimed)"
+                     if wl.features[0].data_type != "float" else ""),
+        "seconds": t, "lookups_per_s": sum(lookups[f] for f in feats) / t,
+    }, {"checked_features": n, "pass": bool(ok), "max_rel_err_beyond_atol": worst}
+
+
+def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: int,
+               grid_blocks: int, cpu_features: int) -> dict:
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import algorithmic_bytes, gen_inputs, gen_tables
+
+    model = pick_model(name)
+    spec = prebuilt.model_spec(model)
+    wl = spec.workload
+    lib_path = prebuilt.ensure_built(model)
+    dev = torch.device("cuda", 0)
+
+    free, total = torch.cuda.mem_get_info(dev)
+    need = wl.table_bytes()
+    if need > free * 0.95:
+        raise RuntimeError(f"{name}: tables need {need / 1e9:.1f} GB, {free / 1e9:.1f} GB free")
+
+    t0 = time.perf_counter()
+    tables = gen_tables(wl, dev)
+    indices, offsets = gen_inputs(wl)
+    d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+    d_off = [torch.from_numpy(o).to(dev) for o in offsets]
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=lib_path)
+    setup_s = time.perf_counter() - t0
+
+    lookups = [len(i) for i in indices]
+    alg_bytes = algorithmic_bytes(wl, lookups)
+
+    run = lambda: layer.forward_indices(d_idx, d_off, tile_bytes=tile_bytes, grid_blocks=grid_blocks)
+    for _ in range(warmup):
+        out = run()
+    torch.cuda.synchronize()
+
+    # K steps bracketed by synchronisation: whole-job rate
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    # per-launch kernel duration with events on the launch stream
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stream = torch.cuda.current_stream(dev)
+    outbuf = torch.empty(wl.batch * wl.embed_dim_sum, dtype=torch.float32, device=dev)
+    for s, e in zip(starts, ends):
+        s.record(stream)
+        layer.lib.process(layer.embed_table_ptrs.data_ptr(), outbuf.data_ptr(), wl.batch,
+                          io_ptrs=layer._io_ptrs.data_ptr(), tile_bytes=tile_bytes,
+                          grid_blocks=grid_blocks, stream=stream.cuda_stream)
+        e.record(stream)
+    torch.cuda.synchronize()
+    durs = sorted(s.elapsed_time(e) * 1e3 for s, e in zip(starts, ends))   # us
+    kernel_us_avg = sum(durs) / len(durs)
+    kernel_us_med = durs[len(durs) // 2]
+
+    res = {
+        "workload": name, "model": model, "features": wl.num_features, "batch": wl.batch,
+        "embed_dim_sum": wl.embed_dim_sum, "lookups": int(sum(lookups)),
+        "table_gb": round(wl.table_bytes() / 1e9, 2),
+        "algorithmic_bytes": int(alg_bytes),
+        "ms_per_step": wall / steps * 1e3,
+        "kernel_us_avg": kernel_us_avg, "kernel_us_median": kernel_us_med,
+        "lookups_per_s": sum(lookups) / (kernel_us_avg * 1e-6),
+        "achieved_gbps": alg_bytes / (kernel_us_avg * 1e-6) / 1e9,
+        "pct_of_peak": alg_bytes / (kernel_us_avg * 1e-6) / 1e9 / HBM_PEAK_GBPS * 100.0,
+        "bodies": layer.lib.info.num_bodies, "occupancy": layer.lib.info.occupancy,
+        "grid_blocks": grid_blocks or layer.max_concurrent_blocks,
+        "setup_s": round(setup_s, 2),
+    }
+    if with_cpu:
+        res["cpu_baseline"], res["check"] = cpu_leg(wl, tables, indices, offsets,
+                                                    out, cpu_features)
+    del layer, tables, d_idx, d_off, out, outbuf
+    torch.cuda.empty_cache()
+    return res
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this path runs on one GPU; --gpus {args.gpus} is not supported "
+              "(the value reported is one GPU's throughput)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the fused kernel has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+
+    if args.copy_calibration > 0:
+        n = args.copy_calibration // 4
+        src = torch.ones(n, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)             # reads n*4 bytes, writes n*4 bytes
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
+
+    head = run_config(args.workload, args.steps, args.warmup, not args.no_cpu, args.tile_bytes,
+                      args.grid_blocks, args.cpu_features)
+    others = {}
+    for name in [n for n in args.also.split(",") if n and n != args.workload]:
+        try:
+            others[name] = run_config(name, args.steps, args.warmup, not args.no_cpu,
+                                      args.tile_bytes, args.grid_blocks, args.cpu_features)
+        except Exception as exc:  # a configuration that does not fit must not hide the headline
+            others[name] = {"error": f"{type(exc).__name__}: {exc}"}
+
+    line = {
+        "metric": METRIC,
+        "value": head["achieved_gbps"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic (seeded; tables N(0,0.01) generated on device)",
+        "config": {"workload": f"{head['workload'].upper()}: {head['features']} features, batch "
+                               f"{head['batch']}, sum(dim) {head['embed_dim_sum']}, "
+                               f"{head['lookups']} lookups, {head['table_gb']} GB of tables",
+                   "model": head["model"], "bodies": head["bodies"],
+                   "occupancy": head["occupancy"], "grid_blocks": head["grid_blocks"]},
+        "kernel_us": head["kernel_us_avg"],
+        "kernel_us_median": head["kernel_us_median"],
+        "lookups_per_s": head["lookups_per_s"],
+        "pct_of_peak": head["pct_of_peak"],
+        "roofline": {"bound": "hbm", "achieved": head["achieved_gbps"], "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": head["achieved_gbps"] / HBM_PEAK_GBPS,
+                     "traffic": None, "kernel": "FusedKnl",
+                     "algorithmic_bytes_per_launch": head["algorithmic_bytes"]},
+    }
+    if "cpu_baseline" in head:
+        line["cpu_baseline"] = head["cpu_baseline"]
+        line["check"] = head["check"]
+    if others:
+        line["configs"] = others
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
