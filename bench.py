@@ -165,9 +165,7 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
     outbuf = torch.empty(wl.batch * wl.embed_dim_sum, dtype=torch.float32, device=dev)
     for s, e in zip(starts, ends):
         s.record(stream)
-        layer.lib.process(layer.embed_table_ptrs.data_ptr(), outbuf.data_ptr(), wl.batch,
-                          io_ptrs=layer._io_ptrs.data_ptr(), tile_bytes=tile_bytes,
-                          grid_blocks=grid_blocks, stream=stream.cuda_stream)
+        layer.forward_indices(d_idx, d_off, tile_bytes=tile_bytes, grid_blocks=grid_blocks, out=outbuf)
         e.record(stream)
     torch.cuda.synchronize()
     durs = sorted(s.elapsed_time(e) * 1e3 for s, e in zip(starts, ends))   # us

@@ -1,0 +1,180 @@
+"""Tune the per-feature schedules and the occupancy of the fused embedding kernel of a model.
+
+    python tune.py -m models/test [-o models/test/output] [-n 8] [-b 256]
+                   [--local_only] [--naive] [--fixed_thread_binding] [--mutation_feat_id K]
+                   [--recompile] [--remeasure] [--noinline] [--debug]
+
+Flags as in the reference's ``examples/tune.py:35-51``.  ``-m`` names a model directory with
+``table_config.txt``, ``schedule_config.txt`` and ``data/`` (``batch_sizes.txt`` + ``f{i}.txt``).
+Additions: ``--workload c3`` tunes one of the built-in synthetic configurations instead of a
+model directory; ``--compile_only`` stops after emitting and building the local-stage kernels
+(no GPU needed -- a later run finds the libraries and only measures); ``--occupancies`` and
+``--sample_batch_nums`` bound the search; ``--profiler events`` times the global stage with
+events instead of spawning rocprofv3.  The result is ``<output>/optimal/`` (sources, library,
+``schedule.json``).
+"""
+
+import argparse
+import json
+import multiprocessing as mp
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import numpy as np
+
+from recflex_amd.tuning import Tuner, TuneConfig, BasicConfig
+from recflex_amd.utils import get_data_fnames
+from recflex_amd.code_emitter.build_basic import BasicBuilder
+
+from schedules.reduce_by_key import ReduceByKeySchedule, ReduceByKeyParams
+from schedules.multi_block_per_sample import MultiBlockPerSampleSchedule, MultiBlockPerSampleParams
+from schedules.one_block_multi_sample import OneBlockMultiSampleSchedule, OneBlockMultiSampleParams
+from schedules.warp_per_sample import WarpPerSampleSchedule, WarpPerSampleParams
+from schedules.one_hot import OneHotSchedule, OneHotParams
+from schedules.one_hot_multi_block import OneHotMultiBlockSchedule, OneHotMultiBlockParams
+from recflex_amd.schedules import (ThreadPerBagSchedule, SubWavefrontPerBagSchedule,
+                                   WavefrontPerBagSchedule, BlockPerBagSchedule)
+
+# number of compute units and resident threads per CU of an MI355X, used when a run only
+# compiles and no device can be queried
+MI355X_CUS = 256
+MI355X_THREADS_PER_CU = 2048
+
+
+def parse_args() -> argparse.Namespace:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("-m", "--model_dir", type=str)
+    parser.add_argument("-o", "--output_dir", type=str)
+    parser.add_argument("-n", "--num_processes", type=int, default=8)
+    parser.add_argument("-b", "--block_threads", type=int, default=256)
+    parser.add_argument("--mutation_feat_id", type=int)
+    parser.add_argument("--naive", action="store_true", default=False)
+    parser.add_argument("--fixed_thread_binding", action="store_true", default=False)
+    parser.add_argument("--thread_binding_choice", type=str, default="mean", choices=["mean", "max"])
+    parser.add_argument("--local_only", action="store_true", default=False)
+    parser.add_argument("--recompile", action="store_true", default=False)
+    parser.add_argument("--remeasure", action="store_true", default=False)
+    parser.add_argument("--noinline", action="store_true", default=False)
+    parser.add_argument("--debug", action="store_true", default=False)
+    parser.add_argument("--workload", type=str, help="built-in synthetic configuration (c1..c5)")
+    parser.add_argument("--workload_batches", type=int, default=2)
+    parser.add_argument("--compile_only", action="store_true", default=False)
+    parser.add_argument("--occupancies", type=str, help="comma-separated workgroups per CU to try")
+    parser.add_argument("--sample_batch_nums", type=int, default=128)
+    parser.add_argument("--profiler", type=str, default="rocprofv3", choices=["rocprofv3", "events"])
+    parser.add_argument("--tile_bytes", type=int, default=0)
+    parser.add_argument("--interference", type=str, default="model", choices=["model", "replicate"],
+                        help="local stage: candidates timed inside the whole model, or per feature "
+                             "against copies of themselves (the reference's scheme)")
+    args = parser.parse_args()
+    if not args.model_dir and not args.workload:
+        parser.error("one of -m/--model_dir and --workload is required")
+    return args
+
+
+def all_templates():
+    return [ThreadPerBagSchedule, SubWavefrontPerBagSchedule, WavefrontPerBagSchedule, BlockPerBagSchedule]
+
+
+def create_tuner(args: argparse.Namespace) -> Tuner:
+    BasicBuilder().build()          # the CPU text front end, once
+    if getattr(args, "workload", None):
+        from recflex_amd.workloads import make_workload, gen_inputs
+        wl = make_workload(args.workload)
+        output_dir = args.output_dir or os.path.join(ROOT, "recflex_amd", "_models", f"tune_{args.workload}")
+        batches = [[] for _ in range(wl.num_features)]
+        for k in range(args.workload_batches):
+            indices, offsets = gen_inputs(wl._replace(seed=wl.seed + 7919 * k))
+            for f in range(wl.num_features):
+                batches[f].append((indices[f], offsets[f]))
+        basic_config = BasicConfig(batch_sizes_fname="", data_fnames=[], schedule_config_fname="",
+                                   table_config_fname="", codegen_dir=output_dir,
+                                   block_threads=args.block_threads,
+                                   sample_batch_nums=args.workload_batches)
+        return Tuner(basic_config, schedule_mapping=globals(), batches=batches,
+                     table_shapes=[(f.rows, f.dim) for f in wl.features],
+                     data_types=[f.data_type for f in wl.features],
+                     schedule_types=[all_templates() for _ in wl.features])
+
+    model_dir = args.model_dir
+    data_dir = os.path.join(model_dir, "data")
+    data_fnames = get_data_fnames(data_dir)
+    output_dir = args.output_dir if args.output_dir else os.path.join(model_dir, "output")
+    basic_config = BasicConfig(batch_sizes_fname=os.path.join(data_dir, "batch_sizes.txt"),
+                               data_fnames=data_fnames,
+                               schedule_config_fname=os.path.join(model_dir, "schedule_config.txt"),
+                               table_config_fname=os.path.join(model_dir, "table_config.txt"),
+                               codegen_dir=output_dir,
+                               block_threads=args.block_threads,
+                               sample_batch_nums=getattr(args, "sample_batch_nums", 128))
+    return Tuner(basic_config=basic_config, schedule_mapping=globals())
+
+
+def create_tune_config(args: argparse.Namespace) -> TuneConfig:
+    try:
+        from recflex_amd.hip_helper import HipInfoQuerier
+        querier = HipInfoQuerier()
+        gpu_ids = querier.gpu_ids
+        sm_count, max_threads_per_sm = querier.get_sm_thread_count()
+    except Exception as exc:
+        if not args.compile_only:
+            raise
+        print(f"no device to query ({exc}); assuming an MI355X for the compile-only run")
+        gpu_ids, sm_count, max_threads_per_sm = [0], MI355X_CUS, MI355X_THREADS_PER_CU
+    if args.occupancies:
+        occupancies = [int(v) for v in args.occupancies.split(",")]
+    else:
+        occupancies = list(range(1, max_threads_per_sm // args.block_threads + 1))
+    kwargs = {}
+    if args.tile_bytes:
+        kwargs["tile_bytes"] = args.tile_bytes
+    return TuneConfig(occupancies=occupancies, gpu_ids=gpu_ids, sm_count=sm_count,
+                      num_processes=args.num_processes, recompile=args.recompile,
+                      remeasure=args.remeasure, inline=not args.noinline, debug=args.debug,
+                      profiler=args.profiler, interference=args.interference, **kwargs)
+
+
+def main():
+    args = parse_args()
+    tuner = create_tuner(args)
+    tune_config = create_tune_config(args)
+
+    if args.compile_only:
+        if tune_config.interference == "model":
+            tuner.compile_tournament(tune_config)
+        else:
+            tuner.compile_local(tune_config)
+        print(f"local-stage kernels built under {tuner.basic.codegen_dir}")
+        return
+
+    if not args.naive:
+        tune_results = tuner.tune(tune_config)
+        print(tune_results)
+        if not args.local_only:
+            occupancy, sched_params = tuner.solve(tune_results, tune_config)
+            print(occupancy, sched_params)
+
+            if args.fixed_thread_binding:
+                fixed_task_blocks, t = tuner.tune_fixed_thread_binding(opt_sched_params=sched_params,
+                                                                       choice=args.thread_binding_choice,
+                                                                       tune_config=tune_config)
+                print(fixed_task_blocks)
+                print(f"Fixed thread binding result: {t/1e6} ms")
+
+            if args.mutation_feat_id is not None and args.mutation_feat_id >= 0:
+                mut_times, opt_idx = tuner.mutation_validation(opt_sched_params=sched_params, opt_occupancy=occupancy,
+                                                               mut_feat_id=args.mutation_feat_id, tune_config=tune_config)
+                print(mut_times, np.argmin(mut_times), opt_idx)
+    else:
+        tune_results, t = tuner.tune_naive(tune_config)
+        print(tune_results)
+        print(f"Naive-tuning result: {t/1e6} ms")
+
+
+if __name__ == "__main__":
+    mp.set_start_method("spawn")
+    main()

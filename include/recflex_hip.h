@@ -52,7 +52,8 @@ typedef struct recom_info {
   int32_t timing;         /* 1 if built with per-feature device timers */
   int32_t tile_bytes;     /* default memory traffic per tile used by the run-time binding */
   int32_t static_binding; /* 1 if the tile count per feature was fixed at emit time */
-  int32_t reserved[7];
+  int32_t num_candidates; /* schedules compiled in; == num_features unless a tuning build */
+  int32_t reserved[6];
 } recom_info;
 
 #define RECOM_ABI_VERSION 1
@@ -68,11 +69,34 @@ int recom_get_info(recom_info *out);
 int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_offsets, int32_t *dtypes,
                              int32_t *row_strides);
 
+/* Number of schedules compiled in for each feature (`num_features` entries): 1 in a production
+ * build; in a tuning build the whole candidate list of the feature, from which each launch
+ * picks one through recom_process_args.d_schedule_choice.  No reference counterpart: the
+ * reference compiles one library per (feature, occupancy) with the candidates laid out as
+ * separate features (RecFlex/tuning/tuner.py:112-126). */
+int recom_get_candidate_counts(int32_t *counts);
+
 /* Workgroups of FusedKnl that are resident at once on the current device
  * (= CUs x workgroups per CU at the emitted occupancy); this is also the size of the
  * persistent grid.  Replaces torch.ops.recom.get_max_concurrent_blocks
  * (RecFlex/code_emitter/codegen.py:446-452, RecFlex/sched_basic_csrc/include/utils.cuh:6-21). */
 int recom_get_max_concurrent_blocks(int32_t *out);
+
+typedef struct recom_launch_info {
+  int32_t compute_units;      /* CUs of the current device */
+  int32_t occupancy;          /* workgroups per CU the persistent grid is sized for */
+  int32_t dyn_lds_bytes;      /* dynamic-LDS pad per workgroup that keeps further ones off a CU */
+  int32_t natural_occupancy;  /* workgroups per CU the kernel's registers and LDS allow */
+  int32_t api_occupancy;      /* hipOccupancyMaxActiveBlocksPerMultiprocessor, for comparison */
+  int32_t num_vgprs;          /* vector registers per lane */
+  int32_t static_lds_bytes;
+  int32_t lds_bytes_per_cu;
+} recom_launch_info;
+
+/* How FusedKnl is launched on the current device: the pieces of the reference's
+ * get_max_concurrent_blocks / get_dyn_smem_size (RecFlex/sched_basic_csrc/include/utils.cuh:6-58),
+ * made visible. */
+int recom_get_launch_info(recom_launch_info *out);
 
 typedef struct recom_process_args {
   /* device int64[F]: base address of each feature's table
@@ -95,6 +119,9 @@ typedef struct recom_process_args {
   int32_t tile_bytes;
   /* persistent grid size; 0 = recom_get_max_concurrent_blocks() */
   int32_t grid_blocks;
+  /* tuning builds: device int32[F], the candidate schedule each feature runs in this launch
+   * (clamped to the feature's candidate count); NULL = candidate 0 everywhere */
+  const int32_t *d_schedule_choice;
   /* timing builds only: device uint64[F], the kernel ADDS each feature's workgroup-ticks
    * (s_memtime) to it; caller zeroes it.  Replaces the per-block clock() array
    * (RecFlex/code_emitter/codegen.py:301-316,388-401).  Must be NULL otherwise. */

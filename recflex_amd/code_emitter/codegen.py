@@ -27,6 +27,8 @@ from .build_basic import BasicBuilder
 
 # memory traffic (bytes) the run-time binding aims at per tile
 DEFAULT_TILE_BYTES = 64 * 1024
+# XCDs (L2 slices) of an MI355X; workgroup i of a launch runs on XCD i % 8
+XCD_COUNT = 8
 # per-bag traffic that does not depend on the bag length, besides the output slice: one offset
 BAG_FIXED_BYTES = 4
 INDEX_BYTES = 4
@@ -41,12 +43,25 @@ def _c_array(ctype: str, name: str, values: List[int], per_line: int = 16) -> st
 
 
 class CodeEmitter:
-    def __init__(self, feat_schedules: List[Tuple[ScheduleBase, NamedTuple]]):
+    def __init__(self, feat_schedules: List[Tuple[ScheduleBase, NamedTuple]],
+                 feat_candidates: List[List[Tuple[ScheduleBase, NamedTuple]]] = None):
+        """``feat_schedules[f]`` is the schedule of feature ``f``.  A tuning build may instead
+        give ``feat_candidates[f]``, the list of schedules feature ``f`` can run; the launch then
+        picks one per feature at run time (``d_schedule_choice``), and ``feat_schedules`` is
+        taken to be each list's first entry."""
+        if feat_candidates is not None:
+            assert all(len(c) > 0 for c in feat_candidates)
+            feat_schedules = [tuple(c[0]) for c in feat_candidates]
         self.feat_schedules: List[Tuple[ScheduleBase, NamedTuple]] = feat_schedules
+        self.feat_candidates = ([[tuple(sp) for sp in c] for c in feat_candidates]
+                                if feat_candidates is not None
+                                else [[tuple(sp)] for sp in feat_schedules])
         if len(self.feat_schedules) > 0:
             self.block_threads: int = feat_schedules[0][0].block_threads
-            for schedule, params in feat_schedules:
-                assert self.block_threads == schedule.block_threads
+            for cands in self.feat_candidates:
+                for schedule, params in cands:
+                    assert self.block_threads == schedule.block_threads
+                    assert schedule.meta == cands[0][0].meta, "candidates of a feature share its table"
 
     # ------------------------------------------------------------------ configuration dump
 
@@ -60,6 +75,9 @@ class CodeEmitter:
             }
             for schedule, params in self.feat_schedules
         ]
+
+    def serialize_candidates(self) -> List[List[Dict[str, Any]]]:
+        return [CodeEmitter(cands).serialize_config() for cands in self.feat_candidates]
 
     def dump_key(self, fname: str) -> None:
         with open(fname, "w") as f:
@@ -84,15 +102,25 @@ class CodeEmitter:
                 return w
         return 1
 
+    def flat_candidates(self) -> Tuple[List[Tuple[ScheduleBase, NamedTuple]], List[int]]:
+        """All candidates in feature order, and ``begin[f]`` = index of feature f's first one."""
+        flat, begin = [], [0]
+        for cands in self.feat_candidates:
+            flat.extend(cands)
+            begin.append(len(flat))
+        return flat, begin
+
     def dedup(self) -> Tuple[Dict[int, int], List[int]]:
-        """feature -> id of the first feature with the same (LDS type, body); list of those ids."""
+        """candidate index -> index of the first candidate with the same (LDS type, body); list
+        of those first indices.  With one schedule per feature, candidate index == feature."""
         seen: Dict[str, int] = {}
         id_map: Dict[int, int] = {}
-        for feat_idx, (schedule, params) in enumerate(self.feat_schedules):
+        flat, _ = self.flat_candidates()
+        for idx, (schedule, params) in enumerate(flat):
             key = schedule.EmitShmemType(params) + "\n" + schedule.EmitScheduleBody(params)
             if key not in seen:
-                seen[key] = feat_idx
-            id_map[feat_idx] = seen[key]
+                seen[key] = idx
+            id_map[idx] = seen[key]
         return id_map, list(seen.values())
 
     # ------------------------------------------------------------------ device code
@@ -106,11 +134,12 @@ class CodeEmitter:
 
     def emit_kernel(self, occupancy: int = None, inline: bool = True, timing: bool = False,
                     timing_branch: bool = False, fixed_task_block_nums: List[int] = None,
-                    tile_bytes: int = None) -> str:
+                    tile_bytes: int = None, xcd_aware: bool = False) -> str:
         num_feats = len(self.feat_schedules)
         assert num_feats > 0, "cannot emit a fused kernel for zero features"
         vars_ = ScheduleVars()
         id_map, body_ids = self.dedup()
+        flat, cand_begin = self.flat_candidates()
         embed_dim_offsets = self.embed_dim_offsets()
 
         consts = f'''constexpr int NUM_FEATS = {num_feats};
@@ -120,6 +149,8 @@ constexpr int {vars_.out_vec} = {self.out_vec()};
 constexpr int OCCUPANCY = {occupancy if occupancy else 0};
 constexpr int TILE_BYTES = {tile_bytes if tile_bytes else DEFAULT_TILE_BYTES};
 constexpr int NUM_BODIES = {len(body_ids)};
+constexpr int NUM_CANDIDATES = {len(flat)};
+constexpr int XCDS = {XCD_COUNT if xcd_aware else 1};
 constexpr bool TIMING = {"true" if timing else "false"};
 constexpr bool STATIC_BINDING = {"true" if fixed_task_block_nums else "false"};
 
@@ -127,8 +158,9 @@ constexpr bool STATIC_BINDING = {"true" if fixed_task_block_nums else "false"};
 
         temp_storage_decl = "union KnlTempStorage {\n"
         functions = ""
+        flat, cand_begin = self.flat_candidates()
         for feat_idx in body_ids:
-            schedule, params = self.feat_schedules[feat_idx]
+            schedule, params = flat[feat_idx]
             temp_storage_decl += f"  {schedule.EmitShmemType(params)} f{feat_idx};\n"
             functions += f'''
 __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{feat_idx}(
@@ -144,14 +176,14 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
 '''
         temp_storage_decl += "};\n\n"
 
-        tables = _c_array("int", "c_process_func_ids", [id_map[f] for f in range(num_feats)])
+        tables = _c_array("int", "c_cand_begin", cand_begin)
+        tables += _c_array("int", "c_cand_func_ids", [id_map[i] for i in range(len(flat))])
+        tables += _c_array("int", "c_cand_gran", [s.TileGranularity(p) for s, p in flat])
         tables += _c_array("int", "c_embed_dim_offsets", embed_dim_offsets)
         tables += _c_array("int", "c_lookup_bytes",
                            [s.meta.row_bytes + INDEX_BYTES for s, _ in self.feat_schedules])
         tables += _c_array("int", "c_bag_bytes",
                            [s.meta.embed_dim * 4 + BAG_FIXED_BYTES for s, _ in self.feat_schedules])
-        tables += _c_array("int", "c_tile_gran",
-                           [s.TileGranularity(p) for s, p in self.feat_schedules])
         if fixed_task_block_nums:
             assert len(fixed_task_block_nums) == num_feats
             tables += _c_array("int", "c_fixed_task_block_nums",
@@ -183,16 +215,29 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     const int64_t *__restrict__ d_arg_buffer_offsets,
     float *__restrict__ d_output,
     const int batch, const int tile_bytes,
+    const int *__restrict__ d_schedule_choice,
     unsigned long long *__restrict__ d_times) {{
   __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;
+
   __shared__ KnlTempStorage s;
 
   const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
   const int total_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}>(
-      s_bind, io, tile_bytes, c_lookup_bytes, c_bag_bytes, c_tile_gran,
-      {"c_fixed_task_block_nums" if fixed_task_block_nums else "nullptr"});
+      s_bind, io, tile_bytes, c_lookup_bytes, c_bag_bytes, c_cand_begin, c_cand_gran,
+      d_schedule_choice, {"c_fixed_task_block_nums" if fixed_task_block_nums else "nullptr"});
 
-  for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {{
+  // Tiles are ordered by feature.  Workgroup i runs on XCD i % XCDS, so the workgroups of one
+  // XCD walk one contiguous 1/XCDS of the tile space: the rows a feature's bags share stay in
+  // that XCD's L2 instead of being fetched into all of them.
+  int tile_first = blockIdx.x, tile_last = total_tiles, tile_step = gridDim.x;
+  if (XCDS > 1 && gridDim.x % XCDS == 0) {{
+    const int chunk = (total_tiles + XCDS - 1) / XCDS;
+    const int xcd = blockIdx.x % XCDS;
+    tile_first = xcd * chunk + blockIdx.x / XCDS;
+    tile_last = min(total_tiles, (xcd + 1) * chunk);
+    tile_step = gridDim.x / XCDS;
+  }}
+  for (int tile = tile_first; tile < tile_last; tile += tile_step) {{
 {timing_begin if timing and timing_branch else ''}
     const int feat_idx = __builtin_amdgcn_readfirstlane(rfx::find_feature<NUM_FEATS>(s_bind, tile));
     const int bags_per_tile = s_bind.bags_per_tile[feat_idx];
@@ -203,7 +248,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     const int *offsets = io.offsets(feat_idx);
     const int embed_dim_offset = c_embed_dim_offsets[feat_idx];
 {timing_begin if timing and not timing_branch else ''}
-    switch (c_process_func_ids[feat_idx]) {{
+    switch (c_cand_func_ids[s_bind.cand[feat_idx]]) {{
 {cases}      default: break;
     }}
 {timing_end}
@@ -234,13 +279,30 @@ extern "C" int recom_process(const recom_process_args *a) {
                      static_cast<hipStream_t>(a->stream),
                      a->d_embed_table_ptrs, a->d_io_ptrs,
                      static_cast<const char *>(a->d_arg_buffers), a->d_arg_buffer_offsets,
-                     a->d_output, a->batch, tile_bytes, a->d_times);
+                     a->d_output, a->batch, tile_bytes, a->d_schedule_choice, a->d_times);
   return static_cast<int>(hipGetLastError());
 }
 '''
 
     def emit_get_concurrent_blocks_func(self, occupancy: int = None) -> str:
         return '''
+extern "C" int recom_get_launch_info(recom_launch_info *out) {
+  if (!out) return static_cast<int>(hipErrorInvalidValue);
+  const rfx::LaunchState *st = nullptr;
+  hipError_t e = rfx::get_launch_state(FusedKnl, BLOCK_THREADS, OCCUPANCY, &st);
+  if (e != hipSuccess) return static_cast<int>(e);
+  *out = recom_launch_info{};
+  out->compute_units = st->cus;
+  out->occupancy = st->occupancy;
+  out->dyn_lds_bytes = st->dyn_lds;
+  out->natural_occupancy = st->natural_occupancy;
+  out->api_occupancy = st->api_occupancy;
+  out->num_vgprs = st->num_vgprs;
+  out->static_lds_bytes = st->static_lds;
+  out->lds_bytes_per_cu = st->lds_per_cu;
+  return static_cast<int>(hipSuccess);
+}
+
 extern "C" int recom_get_max_concurrent_blocks(int32_t *out) {
   if (!out) return static_cast<int>(hipErrorInvalidValue);
   const rfx::LaunchState *st = nullptr;
@@ -265,6 +327,7 @@ extern "C" int recom_get_info(recom_info *out) {
   out->timing = TIMING ? 1 : 0;
   out->tile_bytes = TILE_BYTES;
   out->static_binding = STATIC_BINDING ? 1 : 0;
+  out->num_candidates = NUM_CANDIDATES;
   return 0;
 }
 
@@ -273,6 +336,13 @@ static const int h_embed_dims[] = {H_EMBED_DIMS};
 static const int h_embed_dim_offsets[] = {H_EMBED_DIM_OFFSETS};
 static const int h_dtypes[] = {H_DTYPES};
 static const int h_row_strides[] = {H_ROW_STRIDES};
+static const int h_cand_counts[] = {H_CAND_COUNTS};
+
+extern "C" int recom_get_candidate_counts(int32_t *counts) {
+  if (!counts) return static_cast<int>(hipErrorInvalidValue);
+  for (int f = 0; f < NUM_FEATS; ++f) counts[f] = h_cand_counts[f];
+  return 0;
+}
 
 extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_offsets,
                                         int32_t *dtypes, int32_t *row_strides) {
@@ -287,7 +357,8 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
 '''.replace("H_EMBED_DIMS", ", ".join(map(str, self.embed_dims()))) \
    .replace("H_EMBED_DIM_OFFSETS", ", ".join(map(str, self.embed_dim_offsets()[:-1]))) \
    .replace("H_DTYPES", ", ".join(str(s.meta.dtype_id) for s, _ in self.feat_schedules)) \
-   .replace("H_ROW_STRIDES", ", ".join(str(s.meta.row_stride) for s, _ in self.feat_schedules))
+   .replace("H_ROW_STRIDES", ", ".join(str(s.meta.row_stride) for s, _ in self.feat_schedules)) \
+   .replace("H_CAND_COUNTS", ", ".join(str(len(c)) for c in self.feat_candidates))
 
     # ------------------------------------------------------------------ files
 
@@ -304,7 +375,8 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
 
     def emit(self, ofname: str, occupancy: int = None, inline: bool = True,
              tune: bool = False, timing: bool = False, timing_branch: bool = False,
-             fixed_task_block_nums: List[int] = None, tile_bytes: int = None) -> None:
+             fixed_task_block_nums: List[int] = None, tile_bytes: int = None,
+             xcd_aware: bool = False) -> None:
         """Write the device source.  ``occupancy`` = workgroups per CU the kernel is built and
         launched for (``__launch_bounds__`` budget, persistent grid size, and a dynamic-LDS pad
         that keeps further workgroups off the CU); ``tune`` is accepted for signature
@@ -314,7 +386,7 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
         code += self.emit_kernel(timing=timing, timing_branch=timing_branch,
                                  occupancy=occupancy, inline=inline,
                                  fixed_task_block_nums=fixed_task_block_nums,
-                                 tile_bytes=tile_bytes)
+                                 tile_bytes=tile_bytes, xcd_aware=xcd_aware)
         code += self.emit_process_func(timing=timing, occupancy=occupancy)
         code += self.emit_get_concurrent_blocks_func(occupancy=occupancy)
         code += self.emit_process_ops()

@@ -50,9 +50,14 @@ struct IoView {
   }
 };
 
+// a tile is rounded up to one whole workgroup pass of its schedule only if that pass carries at
+// most this many times the target traffic per tile
+constexpr int kMaxTileFactor = 8;
+
 template <int F> struct BindingStorage {
   int prefix[F + 1];      // prefix[f] = first global tile id of feature f
   int bags_per_tile[F];
+  int cand[F];            // index (into the candidate tables) of the schedule feature f runs
 };
 
 __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
@@ -65,8 +70,11 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
 }
 
 // lookup_bytes[f]: bytes fetched per lookup (row + index); bag_bytes[f]: bytes per bag that do
-// not depend on its length (output row slice + offset); gran[f]: bags a workgroup of this
-// feature's schedule handles per pass (tiles are whole multiples of it).
+// not depend on its length (output row slice + offset).
+// Feature f owns the candidate schedules cand_begin[f] .. cand_begin[f+1]-1 (exactly one in a
+// production build, the whole candidate list in a tuning build); choice[f] (clamped; 0 if
+// choice is null) selects the one this launch runs, and cand_gran[] gives the bags a workgroup
+// of that schedule handles per pass (tiles are whole multiples of it unless a pass is too large).
 // fixed_tiles: if non-null, the tile count per feature is taken from it instead of from the
 // live offsets (static thread binding, for the ablation).
 // Returns the total number of tiles.  Ends with a barrier.
@@ -74,13 +82,19 @@ template <int F, int BT>
 __device__ __forceinline__ int
 bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
            const int *__restrict__ lookup_bytes, const int *__restrict__ bag_bytes,
-           const int *__restrict__ gran, const int *__restrict__ fixed_tiles) {
+           const int *__restrict__ cand_begin, const int *__restrict__ cand_gran,
+           const int *__restrict__ choice, const int *__restrict__ fixed_tiles) {
   const int tid = threadIdx.x;
   const int B = io.batch;
   for (int f = tid; f < F; f += BT) {
-    const int g = gran[f];
-    const int max_tiles = (B + g - 1) / g;
+    const int first = cand_begin[f];
+    const int ncand = cand_begin[f + 1] - first;
+    int pick = choice ? choice[f] : 0;
+    pick = pick < 0 ? 0 : (pick >= ncand ? ncand - 1 : pick);
+    s.cand[f] = first + pick;
+    const int g = cand_gran[first + pick];
     int64_t want;
+    int64_t bag_cost = 0;       // mean traffic of one bag of this feature
     if (fixed_tiles) {
       want = fixed_tiles[f];
     } else {
@@ -88,11 +102,19 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
       const int64_t lookups = static_cast<int64_t>(offs[B]) - offs[0];
       const int64_t cost = lookups * lookup_bytes[f] + static_cast<int64_t>(B) * bag_bytes[f];
       want = (cost + tile_bytes - 1) / tile_bytes;
+      bag_cost = B > 0 ? cost / B : 0;
     }
-    int tiles = want < 1 ? 1 : (want > max_tiles ? max_tiles : static_cast<int>(want));
+    int tiles = want < 1 ? 1 : (want > B ? B : static_cast<int>(want));
     int bpt = 0;
     if (B > 0) {
-      bpt = ((B + tiles - 1) / tiles + g - 1) / g * g;
+      bpt = (B + tiles - 1) / tiles;
+      // Tiles are whole workgroup passes (g bags) -- unless one pass of this schedule is more
+      // than kMaxTileFactor times the traffic a tile should carry: then the tile keeps its
+      // share of the traffic and some of the schedule's teams idle.
+      const int whole = (bpt + g - 1) / g * g;
+      if (fixed_tiles || bpt >= g ||
+          static_cast<int64_t>(whole) * bag_cost <= static_cast<int64_t>(kMaxTileFactor) * tile_bytes)
+        bpt = whole;
       tiles = (B + bpt - 1) / bpt;
     } else {
       tiles = 0;

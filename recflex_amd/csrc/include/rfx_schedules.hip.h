@@ -95,6 +95,58 @@ team_bags(const char *__restrict__ table, const int *__restrict__ indices,
       for (int base = 0; base < len_max; base += U * Y) {
         Vec<VB> buf[UB][U][VPP];
         f32x2 sb[UB][U];
+        const int nbase = base + U * Y;
+
+        // A round in which every lane of the wavefront has all its U lookups: straight-line
+        // code, every load issued before the first add.
+        bool full = true;
+#pragma unroll
+        for (int i = 0; i < UB; ++i) full = full && (beg[i] + nbase <= end[i]);
+        if (__builtin_amdgcn_ballot_w64(!full) == 0) {
+#pragma unroll
+          for (int i = 0; i < UB; ++i)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+              const char *row = table + static_cast<int64_t>(idx[i][u]) * R::STRIDE;
+#pragma unroll
+              for (int v = 0; v < VPP; ++v) {
+                const int c = x + (v0 + v) * X;
+                if (v0 + v < VPL && c < R::V) buf[i][u][v] = load_vec<VB>(row + c * VB);
+              }
+              if constexpr (DT == I8) sb[i][u] = load_scale_bias<D>(row);
+            }
+          // next round's indices: the address is clamped into the bag, the value dropped if
+          // the position lies beyond it
+          int nidx[UB][U];
+#pragma unroll
+          for (int i = 0; i < UB; ++i)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+              const int p = beg[i] + nbase + u * Y + y;
+              nidx[i][u] = indices[p < end[i] ? p : end[i] - 1];
+            }
+#pragma unroll
+          for (int i = 0; i < UB; ++i)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+              for (int v = 0; v < VPP; ++v) {
+                const int c = x + (v0 + v) * X;
+                if (v0 + v < VPL && c < R::V)
+                  accumulate<DT, VB>(acc[i][v], buf[i][u][v], DT == I8 ? sb[i][u].x : 1.f);
+              }
+              if constexpr (DT == I8) bias_acc[i] += sb[i][u].y;
+            }
+#pragma unroll
+          for (int i = 0; i < UB; ++i)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+              const int p = beg[i] + nbase + u * Y + y;
+              idx[i][u] = p < end[i] ? nidx[i][u] : -1;
+            }
+          continue;
+        }
+
 #pragma unroll
         for (int i = 0; i < UB; ++i)
 #pragma unroll
@@ -111,7 +163,6 @@ team_bags(const char *__restrict__ table, const int *__restrict__ indices,
 
         // fetch the next round of indices while the rows are in flight
         int nidx[UB][U];
-        const int nbase = base + U * Y;
 #pragma unroll
         for (int i = 0; i < UB; ++i)
 #pragma unroll

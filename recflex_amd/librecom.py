@@ -24,8 +24,18 @@ class RecomInfo(ctypes.Structure):
         ("timing", ctypes.c_int32),
         ("tile_bytes", ctypes.c_int32),
         ("static_binding", ctypes.c_int32),
-        ("reserved", ctypes.c_int32 * 7),
+        ("num_candidates", ctypes.c_int32),
+        ("reserved", ctypes.c_int32 * 6),
     ]
+
+
+class RecomLaunchInfo(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "compute_units", "occupancy", "dyn_lds_bytes", "natural_occupancy", "api_occupancy",
+        "num_vgprs", "static_lds_bytes", "lds_bytes_per_cu")]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_}
 
 
 class RecomProcessArgs(ctypes.Structure):
@@ -38,13 +48,15 @@ class RecomProcessArgs(ctypes.Structure):
         ("batch", ctypes.c_int32),
         ("tile_bytes", ctypes.c_int32),
         ("grid_blocks", ctypes.c_int32),
+        ("d_schedule_choice", ctypes.c_void_p),
         ("d_times", ctypes.c_void_p),
         ("stream", ctypes.c_void_p),
     ]
 
 
 RECOM_ABI_VERSION = 1
-EXPORTED_SYMBOLS = ("recom_get_info", "recom_get_feature_tables",
+EXPORTED_SYMBOLS = ("recom_get_info", "recom_get_feature_tables", "recom_get_candidate_counts",
+                    "recom_get_launch_info",
                     "recom_get_max_concurrent_blocks", "recom_process")
 
 
@@ -88,6 +100,13 @@ class RecomLib:
         self.embed_dim_offsets: List[int] = list(arrs[1])
         self.dtypes: List[int] = list(arrs[2])
         self.row_strides: List[int] = list(arrs[3])
+        self.lib.recom_get_candidate_counts.restype = ctypes.c_int
+        self.lib.recom_get_candidate_counts.argtypes = [_I32P]
+        counts = (ctypes.c_int32 * f)()
+        rc = self.lib.recom_get_candidate_counts(counts)
+        if rc != 0:
+            raise RecomError("recom_get_candidate_counts", rc)
+        self.candidate_counts: List[int] = list(counts)
 
     @property
     def num_features(self) -> int:
@@ -96,6 +115,15 @@ class RecomLib:
     @property
     def embed_dim_sum(self) -> int:
         return self.info.embed_dim_sum
+
+    def get_launch_info(self) -> RecomLaunchInfo:
+        out = RecomLaunchInfo()
+        self.lib.recom_get_launch_info.restype = ctypes.c_int
+        self.lib.recom_get_launch_info.argtypes = [ctypes.POINTER(RecomLaunchInfo)]
+        rc = self.lib.recom_get_launch_info(ctypes.byref(out))
+        if rc != 0:
+            raise RecomError("recom_get_launch_info", rc)
+        return out
 
     def get_max_concurrent_blocks(self) -> int:
         out = ctypes.c_int32(0)
@@ -106,11 +134,12 @@ class RecomLib:
 
     def process(self, table_ptrs: int, output: int, batch: int, *, io_ptrs: int = 0,
                 arg_buffers: int = 0, arg_buffer_offsets: int = 0, tile_bytes: int = 0,
-                grid_blocks: int = 0, times: int = 0, stream: int = 0) -> None:
+                grid_blocks: int = 0, schedule_choice: int = 0, times: int = 0,
+                stream: int = 0) -> None:
         """All pointer arguments are raw device addresses (``tensor.data_ptr()``)."""
         args = RecomProcessArgs(table_ptrs or None, io_ptrs or None, arg_buffers or None,
                                 arg_buffer_offsets or None, output or None, batch, tile_bytes,
-                                grid_blocks, times or None, stream or None)
+                                grid_blocks, schedule_choice or None, times or None, stream or None)
         rc = self.lib.recom_process(ctypes.byref(args))
         if rc != 0:
             raise RecomError("recom_process", rc)

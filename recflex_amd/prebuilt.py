@@ -6,6 +6,7 @@ its library is missing.  Names:
 
 ``c1`` .. ``c5``     the five benchmark configurations at full size, default (untuned) schedules
 ``c3_tuned``       C3 with the schedules in ``recflex_amd/tuned/c3_schedule.json`` if present
+``c3_xcd``         C3 with the XCD-aware tile walk switched on (for comparison)
 ``c2s`` .. ``c5s``   shrunken C2..C5 (fewer rows / features / samples) that a CPU checker can follow
 ``variants``       one feature per (element type, dim, schedule candidate) over a spread of the
                    candidate space of all four templates, with ragged bags (up to ~1500 lookups)
@@ -35,6 +36,7 @@ class ModelSpec(NamedTuple):
     workload: Workload
     feat_schedules: FeatSchedules
     occupancy: Optional[int]
+    emit_kwargs: dict = {}
 
 
 def metas_of(wl: Workload) -> List[MetaData]:
@@ -45,9 +47,13 @@ def expected_bag_len(f: FeatureSpec) -> float:
     return f.mean_bag * (1.0 - f.empty_frac)
 
 
-def _default(wl: Workload, occupancy: Optional[int] = None) -> ModelSpec:
+# workgroups per CU the untuned models are built for (128 vector registers per lane)
+DEFAULT_OCCUPANCY = 4
+
+
+def _default(wl: Workload, occupancy: Optional[int] = DEFAULT_OCCUPANCY, **emit_kwargs) -> ModelSpec:
     fs = default_feat_schedules(metas_of(wl), [expected_bag_len(f) for f in wl.features], BLOCK_THREADS)
-    return ModelSpec(wl, fs, occupancy)
+    return ModelSpec(wl, fs, occupancy, emit_kwargs)
 
 
 def _tuned(wl: Workload, fname: str) -> ModelSpec:
@@ -92,7 +98,7 @@ def _variants() -> ModelSpec:
                 feats.append(FeatureSpec(int(rng.integers(50, 5000)), dim, data_type, mean, False,
                                          0.1, 1.0))
                 scheds.append((sched, cands[i]))
-    return ModelSpec(Workload("variants", 96, 4242, tuple(feats), "integer"), scheds, None)
+    return ModelSpec(Workload("variants", 96, 4242, tuple(feats), "integer"), scheds, DEFAULT_OCCUPANCY)
 
 
 def _edge() -> ModelSpec:
@@ -101,7 +107,7 @@ def _edge() -> ModelSpec:
     feats = [FeatureSpec(300 + 7 * i, d, t, 5.0, False, 0.2, 0.9) for i, (t, d) in enumerate(dims)]
     wl = Workload("edge", 70, 99, tuple(feats), "integer")
     fs = default_feat_schedules(metas_of(wl), [4.0] * len(feats), BLOCK_THREADS)
-    return ModelSpec(wl, fs, None)
+    return ModelSpec(wl, fs, None)      # no occupancy: natural register use, no LDS pad
 
 
 _SPECS: Dict[str, Callable[[], ModelSpec]] = {
@@ -111,6 +117,7 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c4": lambda: _default(make_workload("C4")),
     "c5": lambda: _default(make_workload("C5")),
     "c3_tuned": lambda: _tuned(make_workload("C3"), "c3_schedule.json"),
+    "c3_xcd": lambda: _default(make_workload("C3"), xcd_aware=True),
     "c2s": lambda: _default(make_workload("C2", batch=512, max_rows=200_000)),
     "c3s": lambda: _default(make_workload("C3", batch=192, max_rows=60_000)),
     "c4s": lambda: _default(make_workload("C4", batch=128, num_features=48, max_rows=30_000)),
@@ -140,7 +147,8 @@ def lib_path(name: str) -> str:
 
 def build(name: str) -> str:
     spec = model_spec(name)
-    return build_model(model_dir(name), spec.feat_schedules, rebuild=True, occupancy=spec.occupancy)
+    return build_model(model_dir(name), spec.feat_schedules, rebuild=True, occupancy=spec.occupancy,
+                       **spec.emit_kwargs)
 
 
 def ensure_built(name: str) -> str:
@@ -150,3 +158,53 @@ def ensure_built(name: str) -> str:
 
 def build_all(names: Optional[List[str]] = None) -> Dict[str, str]:
     return {name: build(name) for name in (names or model_names())}
+
+
+# ------------------------------------------------------------------------------------------------
+# a model directory in the text formats (table_config / schedule_config / data/), built ahead of
+# time the way tune.py and test.py would: local-stage tuning kernels and a default-schedule model
+# ------------------------------------------------------------------------------------------------
+
+TUNE_FIXTURE_OCCUPANCIES = [2, 4]
+TUNE_FIXTURE_SM_COUNT = 256          # compute units of an MI355X
+
+
+def tune_fixture_dir() -> str:
+    return os.path.join(MODELS_DIR, "tune_fixture")
+
+
+def make_fixture_tuner(model_dir: str, sample_batch_nums: int = 4):
+    from .schedules import SCHEDULE_MAPPING
+    from .tuning import BasicConfig, Tuner
+    from .utils import get_data_fnames
+    data_dir = os.path.join(model_dir, "data")
+    cfg = BasicConfig(batch_sizes_fname=os.path.join(data_dir, "batch_sizes.txt"),
+                      data_fnames=get_data_fnames(data_dir),
+                      schedule_config_fname=os.path.join(model_dir, "schedule_config.txt"),
+                      table_config_fname=os.path.join(model_dir, "table_config.txt"),
+                      codegen_dir=tune_fixture_dir(), block_threads=BLOCK_THREADS,
+                      sample_batch_nums=sample_batch_nums)
+    return Tuner(cfg, SCHEDULE_MAPPING)
+
+
+def fixture_tune_config(**overrides):
+    from .tuning import TuneConfig
+    kwargs = dict(occupancies=TUNE_FIXTURE_OCCUPANCIES, gpu_ids=[0], sm_count=TUNE_FIXTURE_SM_COUNT,
+                  num_processes=4, profiler="events", in_process=True)
+    kwargs.update(overrides)
+    return TuneConfig(**kwargs)
+
+
+def build_tune_fixture(model_dir: str) -> str:
+    """Local-stage kernels of the fixture model plus ``default/`` (default schedules, with the
+    generated host front end), all under ``_models/tune_fixture``."""
+    import multiprocessing as mp
+    if mp.get_start_method(allow_none=True) != "spawn":
+        mp.set_start_method("spawn", force=True)
+    tuner = make_fixture_tuner(model_dir)
+    tuner.compile_local(fixture_tune_config(recompile=True, interference="replicate", occupancies=[4]))
+    tuner.compile_tournament(fixture_tune_config(recompile=True, interference="model"))
+    mean_lens = [float(np.mean([len(i) / max(1, len(o) - 1) for i, o in feat])) for feat in tuner.batches]
+    fs = default_feat_schedules(tuner.metas, mean_lens, BLOCK_THREADS)
+    build_model(os.path.join(tune_fixture_dir(), "default"), fs, rebuild=True, occupancy=None)
+    return tune_fixture_dir()

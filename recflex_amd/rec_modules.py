@@ -151,13 +151,26 @@ class FeatEmbed(nn.Module):
     # -------------------------------------------------------------------------------------
 
     def _launch(self, batch: int, timing: bool, timing_schedules: Optional[int], tile_bytes: int,
-                grid_blocks: int, **inputs):
-        output = torch.empty([batch * self.output_units], dtype=torch.float32, device=self.device)
+                grid_blocks: int, schedule_choice: torch.Tensor = None, out: torch.Tensor = None,
+                **inputs):
+        if out is not None:
+            if out.dtype != torch.float32 or out.numel() != batch * self.output_units \
+                    or not out.is_contiguous() or out.device.type != "cuda":
+                raise TypeError(f"out must be a contiguous fp32 device tensor of "
+                                f"{batch * self.output_units} elements")
+            output = out.view(-1)
+        else:
+            output = torch.empty([batch * self.output_units], dtype=torch.float32, device=self.device)
         times = None
         if self.lib.info.timing:
             times = torch.zeros([self.lib.num_features], dtype=torch.int64, device=self.device)
         elif timing:
             raise RuntimeError("timing=True needs a library emitted with timing=True")
+        if schedule_choice is not None:
+            if schedule_choice.dtype != torch.int32 or schedule_choice.numel() != len(self.embed_tables) \
+                    or schedule_choice.device.type != "cuda":
+                raise TypeError("schedule_choice must be an int32 device tensor with one entry per feature")
+            inputs["schedule_choice"] = schedule_choice.data_ptr()
         stream = torch.cuda.current_stream(self.device).cuda_stream
         self.lib.process(self.embed_table_ptrs.data_ptr(), output.data_ptr(), batch,
                          tile_bytes=tile_bytes, grid_blocks=grid_blocks,
@@ -192,10 +205,12 @@ class FeatEmbed(nn.Module):
 
     def forward_indices(self, indices: Sequence[torch.Tensor], offsets: Sequence[torch.Tensor],
                         timing: bool = False, timing_schedules: int = None, tile_bytes: int = 0,
-                        grid_blocks: int = 0):
+                        grid_blocks: int = 0, schedule_choice: torch.Tensor = None,
+                        out: torch.Tensor = None):
         """Per-feature int32 device tensors ``indices[f]`` (``[L_f]``) and ``offsets[f]``
         (``[batch + 1]``, exclusive prefix sums, ``offsets[f][0] == 0``) -> ``[batch, sum(dim)]``
-        fp32 (with ``timing=True``: ``(output, task_times)``)."""
+        fp32 (with ``timing=True``: ``(output, task_times)``).  ``out``: write into this
+        preallocated tensor instead of allocating one."""
         n = len(self.embed_tables)
         if len(indices) != n or len(offsets) != n:
             raise ValueError(f"expected {n} index and offset tensors")
@@ -214,6 +229,7 @@ class FeatEmbed(nn.Module):
             self._io_ptrs = torch.tensor(flat, dtype=torch.int64, device=self.device)
             self._io_cache_key = key
         res = self._launch(batch, timing, timing_schedules, tile_bytes, grid_blocks,
+                           schedule_choice=schedule_choice, out=out,
                            io_ptrs=self._io_ptrs.data_ptr())
         if timing:
             return res[0].view(batch, self.output_units), res[1]

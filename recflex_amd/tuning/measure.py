@@ -1,0 +1,341 @@
+"""Measurement workers of the tuner.
+
+Function names and roles follow ``RecFlex/tuning/measure.py:20-122``:
+
+* ``measure_single_feat``   local stage: every candidate schedule of one feature runs as its own
+  "feature" of one fused kernel over the same data (replicated until the GPU is full, which is
+  the simulated interference); the kernel is a timing build, and the time of a candidate is the
+  sum of the device ticks of its tiles.  Writes ``result.txt`` (space separated floats)
+  atomically.
+* ``measure_naive_candidate``  one candidate alone on the GPU, timed with events.
+* ``rocprof_profile``       global stage: run ``run_script.py`` under
+  ``rocprofv3 --kernel-trace --stats`` (the reference uses ``nsys profile``) and leave the
+  kernel statistics next to the build.
+* ``measure_kernel_events`` the same quantity without an external profiler (events around each
+  launch), for machines where spawning the profiler is not wanted.
+* ``measure_task_blocks``   tiles per feature and batch under the run-time binding (input of
+  the fixed-thread-binding ablation).
+
+A worker may run in a spawned process pinned to one GPU (``gpu_id`` keyword, set through
+``HIP_VISIBLE_DEVICES``) or be called directly: emitted libraries are plain ``dlopen`` handles,
+so one process can measure any number of them -- the reference needs a process per library
+because ``TORCH_LIBRARY(recom)`` can be registered once (``measure.py:23-24``).
+"""
+
+import json
+import os
+import shutil
+import subprocess
+import sys
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+
+
+def _pin_gpu(gpu_id: Optional[int]) -> None:
+    if gpu_id is None:
+        raise Exception("No valid GPU provided!")
+    # only effective before the HIP runtime starts, i.e. in a freshly spawned worker
+    if "torch" not in sys.modules:
+        os.environ["HIP_VISIBLE_DEVICES"] = str(gpu_id)
+
+
+def load_batches(data_npz: str) -> List[Tuple[np.ndarray, np.ndarray]]:
+    """``[(indices, offsets)]`` of one feature, as written by ``save_batches``."""
+    z = np.load(data_npz)
+    n = int(z["num_batches"])
+    return [(z[f"indices{k}"], z[f"offsets{k}"]) for k in range(n)]
+
+
+def save_batches(data_npz: str, batches: Sequence[Tuple[np.ndarray, np.ndarray]]) -> None:
+    arrays = {"num_batches": np.int64(len(batches))}
+    for k, (idx, off) in enumerate(batches):
+        arrays[f"indices{k}"] = np.asarray(idx, dtype=np.int32)
+        arrays[f"offsets{k}"] = np.asarray(off, dtype=np.int32)
+    tmp = data_npz + ".tmp.npz"
+    np.savez(tmp, **arrays)
+    os.replace(tmp, data_npz)
+
+
+def make_table(table_shape: Tuple[int, int], data_type: str, device, ones: bool = True):
+    """Table of the right storage type; ``ones`` as in the reference's tuning runs
+    (``measure.py:41``), else N(0, 1)."""
+    import torch
+    from recflex_amd.quant import quantize_rowwise_int8
+    rows, dim = table_shape
+    w = torch.ones(rows, dim, dtype=torch.float32, device=device) if ones else \
+        torch.randn(rows, dim, dtype=torch.float32, device=device)
+    if data_type == "half":
+        return w.half()
+    if data_type == "int8":
+        return quantize_rowwise_int8(w)
+    return w
+
+
+def _write_atomically(path: str, text: str) -> None:
+    tmp = path + ".tmp"
+    with open(tmp, "w") as f:
+        f.write(text)
+    os.replace(tmp, path)
+
+
+def measure_single_feat(ident: Tuple[int, int], data_npz: str, table_shape: Tuple[int, int],
+                        data_type: str, num_schedules: int, num_padded_schedules: int,
+                        librecom_path: str, output_path: str, gpu_id: int = None) -> Optional[List[float]]:
+    feat_id, occupancy = ident
+    print(f"Feat {feat_id}, Occ {occupancy}, GPU {gpu_id}", flush=True)
+    try:
+        _pin_gpu(gpu_id)
+        import torch
+        assert torch.cuda.is_available()
+        from recflex_amd.rec_modules import FeatEmbed
+
+        dev = torch.device("cuda", torch.cuda.current_device())
+        table = make_table(table_shape, data_type, dev)
+        layer = FeatEmbed(dev, embed_tables=[table for _ in range(num_padded_schedules)],
+                          librecom=librecom_path)
+        accum = torch.zeros([num_schedules], dtype=torch.float64)
+        for idx, off in load_batches(data_npz):
+            d_idx = torch.from_numpy(idx).to(dev)
+            d_off = torch.from_numpy(off).to(dev)
+            _, task_times = layer.forward_indices([d_idx] * num_padded_schedules,
+                                                  [d_off] * num_padded_schedules,
+                                                  timing=True, timing_schedules=num_schedules)
+            accum += task_times
+        torch.cuda.synchronize()
+        result = [t.item() for t in accum]
+        _write_atomically(output_path, ' '.join(str(t) for t in result))
+        return result
+    except Exception as e:  # a failed worker leaves no result file; the tuner notices that
+        print(f"[{ident}] Exception {type(e).__name__}: {e}", flush=True)
+        return None
+
+
+def measure_tournament(ident: int, librecom_path: str, table_shapes: Sequence[Tuple[int, int]],
+                       data_types: Sequence[str], data_npzs: Sequence[str], output_path: str,
+                       rounds: int = 3, refine_passes: int = 3, top_k: int = 8,
+                       probe_fraction: float = 0.2, probes_per_candidate: int = 3, seed: int = 0,
+                       gpu_id: int = None) -> Optional[List[List[float]]]:
+    """Local stage inside the real model: the library holds every candidate of every feature
+    and each launch runs one candidate per feature (``d_schedule_choice``), so a candidate is
+    timed against the memory traffic of all the other features, not against copies of itself.
+
+    Exploration: ``rounds`` times, every feature walks a random permutation of its candidates
+    (one launch per step, all features step together); a candidate's score is its mean summed
+    tile time.  Refinement, ``refine_passes`` times: every feature runs its current best except a
+    random ``probe_fraction`` of the features, each of which tries one of its ``top_k``
+    candidates; the scores measured against this near-final background replace the exploration
+    scores of those candidates and the best is re-elected.  Writes
+    ``{"times": [[score per candidate] per feature], "best": [...]}`` as JSON."""
+    print(f"Tournament, Occ {ident}, GPU {gpu_id}", flush=True)
+    try:
+        _pin_gpu(gpu_id)
+        import torch
+        assert torch.cuda.is_available()
+        from recflex_amd.rec_modules import FeatEmbed
+
+        dev = torch.device("cuda", torch.cuda.current_device())
+        tables = [make_table(s, t, dev, ones=False) for s, t in zip(table_shapes, data_types)]
+        layer = FeatEmbed(dev, embed_tables=tables, librecom=librecom_path)
+        counts = layer.lib.candidate_counts
+        num_feats = len(counts)
+        per_feat = [load_batches(p) for p in data_npzs]
+        device_batches = []
+        for k in range(len(per_feat[0])):
+            device_batches.append(([torch.from_numpy(b[k][0]).to(dev) for b in per_feat],
+                                   [torch.from_numpy(b[k][1]).to(dev) for b in per_feat]))
+        rng = np.random.default_rng(seed)
+
+        def launch(choice: np.ndarray) -> np.ndarray:
+            d_choice = torch.from_numpy(choice.astype(np.int32)).to(dev)
+            total = np.zeros(num_feats, dtype=np.float64)
+            for d_idx, d_off in device_batches:
+                _, t = layer.forward_indices(d_idx, d_off, timing=True, schedule_choice=d_choice)
+                total += t.numpy()
+            return total
+
+        launch(np.zeros(num_feats, dtype=np.int32))      # warm-up
+        # ---- exploration
+        sums = [np.zeros(c) for c in counts]
+        hits = [np.zeros(c) for c in counts]
+        steps = max(counts)
+        for _ in range(rounds):
+            perms = [rng.permutation(c) for c in counts]
+            for j in range(steps):
+                choice = np.array([perms[f][j % counts[f]] for f in range(num_feats)])
+                t = launch(choice)
+                for f in range(num_feats):
+                    sums[f][choice[f]] += t[f]
+                    hits[f][choice[f]] += 1
+        score = [s / np.maximum(h, 1) for s, h in zip(sums, hits)]
+        best = np.array([int(np.argmin(sc)) for sc in score])
+
+        # ---- refinement against the incumbent mix
+        for _ in range(refine_passes):
+            tops = [np.argsort(sc)[:min(top_k, len(sc))] for sc in score]
+            rsum = [np.zeros(c) for c in counts]
+            rhit = [np.zeros(c) for c in counts]
+            launches = int(np.ceil(max(len(t) for t in tops) * probes_per_candidate / probe_fraction))
+            for _ in range(launches):
+                choice = best.copy()
+                probing = rng.random(num_feats) < probe_fraction
+                for f in np.nonzero(probing)[0]:
+                    choice[f] = rng.choice(tops[f])
+                t = launch(choice)
+                for f in range(num_feats):
+                    rsum[f][choice[f]] += t[f]
+                    rhit[f][choice[f]] += 1
+            for f in range(num_feats):
+                seen = rhit[f] > 0
+                refined = np.where(seen, rsum[f] / np.maximum(rhit[f], 1), np.inf)
+                worst_seen = refined[seen].max() if seen.any() else 0.0
+                # candidates not re-measured keep their exploration score, but never beat a
+                # candidate that was measured against the incumbent mix
+                score[f] = np.where(seen, refined, np.maximum(score[f], worst_seen))
+                best[f] = int(np.argmin(score[f]))
+        torch.cuda.synchronize()
+        result = [sc.tolist() for sc in score]
+        _write_atomically(output_path, json.dumps({"times": result, "best": best.tolist()}))
+        return result
+    except Exception as e:
+        print(f"[tournament {ident}] Exception {type(e).__name__}: {e}", flush=True)
+        return None
+
+
+def measure_naive_candidate(ident: Tuple[int, int], data_npz: str, table_shape: Tuple[int, int],
+                            data_type: str, librecom_path: str, output_path: str,
+                            gpu_id: int = None) -> Optional[float]:
+    feat_id, sched_param_id = ident
+    print(f"Feat {feat_id}, Schedule {sched_param_id}, GPU {gpu_id}", flush=True)
+    try:
+        _pin_gpu(gpu_id)
+        import torch
+        assert torch.cuda.is_available()
+        from recflex_amd.rec_modules import FeatEmbed
+
+        dev = torch.device("cuda", torch.cuda.current_device())
+        layer = FeatEmbed(dev, embed_tables=[make_table(table_shape, data_type, dev)],
+                          librecom=librecom_path)
+        accum_ms = 0.0
+        for idx, off in load_batches(data_npz):
+            d_idx = [torch.from_numpy(idx).to(dev)]
+            d_off = [torch.from_numpy(off).to(dev)]
+            layer.forward_indices(d_idx, d_off)          # warm-up (first launch sets the grid up)
+            start = torch.cuda.Event(enable_timing=True)
+            end = torch.cuda.Event(enable_timing=True)
+            start.record()
+            layer.forward_indices(d_idx, d_off)
+            end.record()
+            end.synchronize()
+            accum_ms += start.elapsed_time(end)
+        _write_atomically(output_path, str(accum_ms))
+        return accum_ms
+    except Exception as e:
+        print(f"[{ident}] Exception {type(e).__name__}: {e}", flush=True)
+        return None
+
+
+def _run_script_args(table_config_fname: str, build_dir: str, data_dir: str,
+                     sample_batch_nums: int, spec_feat_id: Optional[int]) -> List[str]:
+    script_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "run_script.py")
+    args = [sys.executable, script_path, "--table_config_fname", table_config_fname,
+            "--build_dir", build_dir, "--data_dir", data_dir,
+            "--sample_batch_nums", str(sample_batch_nums)]
+    if spec_feat_id is not None:
+        args += ["--spec_feat_id", str(spec_feat_id)]
+    return args
+
+
+def rocprof_profile(table_config_fname: str, build_dir: str, data_dir: str, sample_batch_nums: int,
+                    report_prefix: str, spec_feat_id: int = None, gpu_id: int = None) -> None:
+    """Leaves ``{report_prefix}_kernel_stats.csv`` (rocprofv3 ``--kernel-trace --stats``)."""
+    if gpu_id is None:
+        raise Exception("No valid GPU provided!")
+    rocprof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    out_dir = os.path.dirname(os.path.abspath(report_prefix))
+    name = os.path.basename(report_prefix)
+    cmd = [rocprof, "--kernel-trace", "--stats", "--output-format", "csv", "-d", out_dir, "-o", name,
+           "--"] + _run_script_args(table_config_fname, build_dir, data_dir, sample_batch_nums,
+                                    spec_feat_id)
+    env = dict(os.environ)
+    env["HIP_VISIBLE_DEVICES"] = str(gpu_id)
+    env.setdefault("TMPDIR", "/tmp")
+    # like nsys in the reference, the profiler's own exit status is not trusted; the stats file is
+    subprocess.run(cmd, env=env, cwd="/tmp", stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+
+
+# the reference's name for the global-stage worker
+nsys_profile = rocprof_profile
+
+
+def measure_kernel_events(librecom_path: str, table_shapes: Sequence[Tuple[int, int]],
+                          data_types: Sequence[str], data_npzs: Sequence[str], output_path: str,
+                          repeats: int = 20, warmup: int = 10, gpu_id: int = None) -> Optional[float]:
+    """Total FusedKnl time in ns over all batches (median of ``repeats`` launches per batch),
+    measured with events on the launch stream; written to ``output_path``."""
+    try:
+        _pin_gpu(gpu_id)
+        import torch
+        from recflex_amd.rec_modules import FeatEmbed
+
+        dev = torch.device("cuda", torch.cuda.current_device())
+        tables = [make_table(s, t, dev, ones=False) for s, t in zip(table_shapes, data_types)]
+        layer = FeatEmbed(dev, embed_tables=tables, librecom=librecom_path)
+        per_feat = [load_batches(p) for p in data_npzs]
+        total_ns = 0.0
+        for k in range(len(per_feat[0])):
+            d_idx = [torch.from_numpy(b[k][0]).to(dev) for b in per_feat]
+            d_off = [torch.from_numpy(b[k][1]).to(dev) for b in per_feat]
+            out = layer.forward_indices(d_idx, d_off)       # its buffer is reused below
+            for _ in range(warmup):                         # let the clocks settle
+                layer.forward_indices(d_idx, d_off, out=out)
+            times = []
+            for _ in range(repeats):
+                start = torch.cuda.Event(enable_timing=True)
+                end = torch.cuda.Event(enable_timing=True)
+                start.record()
+                layer.forward_indices(d_idx, d_off, out=out)
+                end.record()
+                end.synchronize()
+                times.append(start.elapsed_time(end) * 1e6)
+            total_ns += sorted(times)[len(times) // 2]
+        _write_atomically(output_path, str(total_ns))
+        return total_ns
+    except Exception as e:
+        print(f"[{librecom_path}] Exception {type(e).__name__}: {e}", flush=True)
+        return None
+
+
+MAX_TILE_FACTOR = 8      # rfx::kMaxTileFactor
+
+
+def tiles_per_feature(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int],
+                      bag_bytes: Sequence[int], gran: Sequence[int], tile_bytes: int) -> List[int]:
+    """Host restatement of the device binding (``rfx::bind_tiles``): tiles each feature gets
+    for this batch."""
+    out = []
+    for off, lb, bb, g in zip(offsets, lookup_bytes, bag_bytes, gran):
+        batch = len(off) - 1
+        if batch <= 0:
+            out.append(0)
+            continue
+        cost = int(off[-1] - off[0]) * lb + batch * bb
+        tiles = min(max(-(-cost // tile_bytes), 1), batch)
+        bpt = -(-batch // tiles)
+        whole = -(-bpt // g) * g
+        if bpt >= g or whole * (cost // batch) <= MAX_TILE_FACTOR * tile_bytes:
+            bpt = whole
+        out.append(-(-batch // bpt))
+    return out
+
+
+def measure_task_blocks(data_npzs: Sequence[str], lookup_bytes: Sequence[int],
+                        bag_bytes: Sequence[int], gran: Sequence[int], tile_bytes: int,
+                        output_path: str) -> None:
+    """One line per batch: comma separated tile counts per feature (CPU only)."""
+    per_feat = [load_batches(p) for p in data_npzs]
+    lines = []
+    for k in range(len(per_feat[0])):
+        tiles = tiles_per_feature([b[k][1] for b in per_feat], lookup_bytes, bag_bytes, gran, tile_bytes)
+        lines.append(','.join(str(t) for t in tiles))
+    _write_atomically(output_path, '\n'.join(lines) + '\n')

@@ -1,0 +1,574 @@
+"""Two-stage, interference-aware schedule tuner for CDNA4.
+
+Class, method and field names follow ``RecFlex/tuning/tuner.py:24-357`` (``BasicConfig``,
+``TuneConfig``, ``Tuner.tune`` / ``solve`` / ``tune_occupancy`` / ``mutation_validation`` /
+``tune_naive`` / ``tune_fixed_thread_binding`` / ``emit_codes``), and so does the output tree
+under ``codegen_dir``: ``f{feat}/o{occ}/``, ``all/o{occ}/``, ``optimal/``, ``naive/``,
+``mutation_f{id}/m{k}``, ``fixed_thread_binding_{mean,max}/``, with ``result.txt`` files and the
+resume-by-files rule (an existing ``librecom.so`` / result is kept unless ``recompile`` /
+``remeasure``).
+
+Local stage: for every feature and occupancy, all candidate schedules of the feature are put
+side by side as the "features" of one fused kernel, repeated until there are at least
+``CUs * occupancy`` of them, over the same input data; the kernel is built for exactly
+``occupancy`` workgroups per CU (``__launch_bounds__`` register budget + dynamic-LDS pad +
+persistent grid of ``CUs * occupancy`` workgroups) with per-feature device timers; the candidate
+with the smallest summed tile time wins.  Global stage: per occupancy, the whole model with the
+winners is built and its ``FusedKnl`` time measured (rocprofv3 kernel statistics, or events);
+the fastest occupancy is copied to ``optimal/`` together with ``optimal/schedule.json``.
+
+CDNA4 specifics: occupancy is counted in 256-thread workgroups per CU (= wavefronts per SIMD),
+1..8.  Kernels whose candidate lists are identical (features with the same dim and element type)
+are compiled once and shared through ``.cache/``.
+"""
+
+import hashlib
+import json
+import os
+import shutil
+from typing import Dict, List, NamedTuple, Optional, Sequence, Tuple
+
+import numpy as np
+
+from recflex_amd.code_emitter import CodeEmitter, ScheduleBase, MetaData
+from recflex_amd.code_emitter.codegen import BAG_FIXED_BYTES, DEFAULT_TILE_BYTES, INDEX_BYTES
+from recflex_amd.utils import find_file, compile_build, os_check
+from recflex_amd.task_manager import TaskManager
+from recflex_amd.parser import (parse_raw_data_batches, parse_table_shapes, parse_table_dtypes,
+                                parse_schedule_types, parse_knl_total_time)
+
+from .measure import (measure_single_feat, rocprof_profile, measure_task_blocks,
+                      measure_naive_candidate, measure_kernel_events, measure_tournament,
+                      save_batches)
+
+
+class BasicConfig(NamedTuple):
+    batch_sizes_fname: str
+    data_fnames: List[str]
+    schedule_config_fname: str
+    table_config_fname: str
+    codegen_dir: str
+    subdirs: List[str] = []
+    includes: List[str] = []
+    links: List[str] = []
+    host_links: List[str] = []
+    block_threads: int = 256
+    sample_batch_nums: int = 128
+
+
+class TuneConfig(NamedTuple):
+    occupancies: List[int]
+    gpu_ids: List[int]
+    sm_count: int
+    num_processes: int = 8
+    inline: bool = True
+    recompile: bool = False
+    remeasure: bool = False
+    debug: bool = False
+    # "rocprofv3": global-stage kernel time from rocprofv3 kernel statistics (spawned);
+    # "events": events around each launch, in this process
+    profiler: str = "rocprofv3"
+    # run measurement workers in this process instead of one spawned process per measurement
+    in_process: bool = True
+    tile_bytes: int = DEFAULT_TILE_BYTES
+    # local-stage interference: "model" = every candidate of every feature is compiled into one
+    # kernel of the whole model and timed while all other features run beside it;
+    # "replicate" = per feature, the candidates side by side over the same data, replicated
+    # until the GPU is full (the reference's scheme, RecFlex/tuning/tuner.py:112-141)
+    interference: str = "model"
+    rounds: int = 3
+    refine_passes: int = 3
+    top_k: int = 8
+
+
+def padded_sched_num(orig_num: int, max_concurrent_blocks: int) -> int:
+    return (orig_num + max_concurrent_blocks - 1) // orig_num * orig_num
+
+
+class Tuner:
+    def __init__(self, basic_config: BasicConfig, schedule_mapping: Dict[str, type],
+                 batches: List[List[Tuple[np.ndarray, np.ndarray]]] = None,
+                 table_shapes: List[Tuple[int, int]] = None, data_types: List[str] = None,
+                 schedule_types: List[List[type]] = None):
+        """With only ``basic_config`` and ``schedule_mapping`` everything is read from the files
+        the configuration names, as in the reference.  The keyword arguments supply the same
+        information directly (synthetic workloads that have no dataset directory):
+        ``batches[feat][k] = (indices, offsets)``."""
+        self.basic = basic_config
+        self.schedule_mapping = schedule_mapping
+        self._given = (batches, table_shapes, data_types, schedule_types)
+        self.get_raw_data_batches()
+        self.get_metas()
+        self.get_feat_schedules()
+        self.num_feats: int = len(self.feat_schedules)
+        self.gen_feat_sched_param_candidates()
+        self.write_data_files()
+
+    # ------------------------------------------------------------------ inputs
+
+    def get_raw_data_batches(self):
+        """``self.batches[feat]`` = list of ``(indices, offsets)`` int32 arrays, one per sampled
+        batch; ``self.raw_data_batches`` keeps the text lines when they came from files."""
+        given = self._given[0]
+        if given is not None:
+            self.raw_data_batches = None
+            self.batches = given
+            return self.batches
+        from recflex_amd.host import RecomHost
+        self.raw_data_batches = parse_raw_data_batches(self.basic.batch_sizes_fname,
+                                                       self.basic.data_fnames,
+                                                       self.basic.sample_batch_nums)
+        host = RecomHost()
+        self.batches = [[host.parse_lines(lines) for lines in feat] for feat in self.raw_data_batches]
+        return self.raw_data_batches
+
+    def get_metas(self):
+        _, shapes, dtypes, _ = self._given
+        self.table_shapes = shapes if shapes is not None else parse_table_shapes(self.basic.table_config_fname)
+        if dtypes is not None:
+            self.data_types = list(dtypes)
+        elif shapes is None:
+            self.data_types = parse_table_dtypes(self.basic.table_config_fname)
+        else:
+            self.data_types = ["float"] * len(self.table_shapes)
+        self.metas: List[MetaData] = [MetaData(embed_dim=embed_dim, data_type=dt)
+                                      for (nrows, embed_dim), dt in zip(self.table_shapes, self.data_types)]
+        return self.metas
+
+    def get_feat_schedules(self):
+        feat_schedule_types = self._given[3]
+        if feat_schedule_types is None:
+            feat_schedule_types = parse_schedule_types(self.basic.schedule_config_fname, self.schedule_mapping)
+        for f, types in enumerate(feat_schedule_types):
+            if any(t is None for t in types):
+                raise KeyError(f"feature {f}: unknown schedule class name in the schedule config")
+        self.feat_schedules: List[List[ScheduleBase]] = [
+            [schedule_type(meta, self.basic.block_threads) for schedule_type in schedule_types]
+            for schedule_types, meta in zip(feat_schedule_types, self.metas)]
+        return self.feat_schedules
+
+    def gen_feat_sched_param_candidates(self):
+        self.feat_sched_param_candidates: List[List[Tuple[ScheduleBase, NamedTuple]]] = [[] for _ in range(self.num_feats)]
+        for feat_id in range(self.num_feats):
+            for schedule in self.feat_schedules[feat_id]:
+                for params in schedule.GenParamCandidates():
+                    self.feat_sched_param_candidates[feat_id].append([schedule, params])
+            if not self.feat_sched_param_candidates[feat_id]:
+                raise ValueError(f"feature {feat_id}: its schedule classes produced no candidate")
+
+    def write_data_files(self):
+        """Per-feature ``data/f{i}.npz`` under ``codegen_dir`` (what the workers read) and, for
+        workloads given as arrays, a ``table_config.txt`` for the profiling driver."""
+        self.data_dir = f"{self.basic.codegen_dir}/data"
+        os.makedirs(self.data_dir, exist_ok=True)
+        self.data_npzs = []
+        for feat_id in range(self.num_feats):
+            path = f"{self.data_dir}/f{feat_id}.npz"
+            save_batches(path, self.batches[feat_id])
+            self.data_npzs.append(path)
+        self.table_config_fname = self.basic.table_config_fname
+        if not self.table_config_fname or not os.path.exists(self.table_config_fname):
+            self.table_config_fname = f"{self.data_dir}/table_config.txt"
+            with open(self.table_config_fname, "w") as f:
+                for (rows, dim), dt in zip(self.table_shapes, self.data_types):
+                    f.write(f"{rows},{dim},{dt}\n")
+
+    # ------------------------------------------------------------------ helpers
+
+    def get_padded_sched_num(self, orig_num: int, max_concurrent_blocks: int) -> int:
+        return padded_sched_num(orig_num, max_concurrent_blocks)
+
+    def pad_sched_params(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]], padded_num: int) -> List[Tuple[ScheduleBase, NamedTuple]]:
+        padded_schedules = sched_params.copy()
+        add_num = padded_num - len(sched_params)
+        for i in range(add_num):
+            padded_schedules.append(sched_params[i % len(sched_params)])
+        return padded_schedules
+
+    def get_output_build_dir(self, feat_id: int, occupancy: int) -> Tuple[str, str]:
+        if feat_id >= 0:
+            output_dir = f"{self.basic.codegen_dir}/f{feat_id}/o{occupancy}"
+        else:
+            output_dir = f"{self.basic.codegen_dir}/all/o{occupancy}"
+        build_dir = f"{output_dir}/build"
+        return output_dir, build_dir
+
+    def emit_codes(self, output_dir: str, feat_schedules: List[Tuple[ScheduleBase, NamedTuple]],
+                   occupancy: int, inline: bool = True, timing: bool = False, tune: bool = False,
+                   fixed_task_block_nums: List[int] = None, debug: bool = False,
+                   tile_bytes: int = None, host: bool = True) -> None:
+        os.makedirs(output_dir, exist_ok=True)
+        emitter = CodeEmitter(feat_schedules)
+        if host:
+            emitter.emit_host(f"{output_dir}/preprocess.cpp", fixed_task_block_nums=fixed_task_block_nums)
+        emitter.emit(f"{output_dir}/process.hip", occupancy=occupancy, timing=timing, inline=inline, tune=tune,
+                     fixed_task_block_nums=fixed_task_block_nums, tile_bytes=tile_bytes)
+        emitter.emit_cmake_list(f"{output_dir}/CMakeLists.txt", code_fname="process.hip",
+                                host_fname="preprocess.cpp" if host else None,
+                                subdirs=self.basic.subdirs, includes=self.basic.includes, links=self.basic.links,
+                                host_links=self.basic.host_links, debug=debug)
+        if not tune:      # local-stage kernels are candidate lists, not a model's schedule
+            emitter.dump_key(f"{output_dir}/schedule.json")
+
+    # ---- compile cache: identical device sources are built once -----------------------------
+
+    def _source_key(self, output_dir: str) -> str:
+        with open(f"{output_dir}/process.hip", "rb") as f:
+            return hashlib.sha256(f.read()).hexdigest()[:24]
+
+    def _cached_lib(self, key: str) -> str:
+        return f"{self.basic.codegen_dir}/.cache/{key}/librecom.so"
+
+    def _schedule_builds(self, jobs: List[Tuple[str, str]], tune_config: TuneConfig) -> None:
+        """``jobs`` = (output_dir, build_dir) whose sources are emitted.  Builds each distinct
+        source once (in parallel worker processes), then links every build dir to its library."""
+        by_key: Dict[str, List[Tuple[str, str]]] = {}
+        for output_dir, build_dir in jobs:
+            by_key.setdefault(self._source_key(output_dir), []).append((output_dir, build_dir))
+        to_publish = []
+        for key, group in by_key.items():
+            if os.path.exists(self._cached_lib(key)) and not tune_config.recompile:
+                continue
+            to_publish.append((key, group[0][1]))
+        if to_publish:
+            manager = TaskManager(list(range(max(1, tune_config.num_processes))))
+            for key, build_dir in to_publish:
+                os.makedirs(build_dir, exist_ok=True)
+                manager.add_task(compile_build, (build_dir,))
+            manager.join()
+        for key, build_dir in to_publish:
+            lib = f"{build_dir}/librecom.so"
+            if not os.path.exists(lib):
+                raise Exception(f"build failed: {lib} was not produced")
+            os.makedirs(os.path.dirname(self._cached_lib(key)), exist_ok=True)
+            shutil.copyfile(lib, self._cached_lib(key))
+        for key, group in by_key.items():
+            for output_dir, build_dir in group:
+                os.makedirs(build_dir, exist_ok=True)
+                self._link_lib(self._cached_lib(key), f"{build_dir}/librecom.so")
+
+    @staticmethod
+    def _link_lib(src: str, dst: str) -> None:
+        """Make ``dst`` the same file as ``src`` (hard link; a copy where links are refused)."""
+        if os.path.exists(dst) and os.path.samefile(src, dst):
+            return
+        tmp = dst + ".tmp"
+        if os.path.exists(tmp):
+            os.remove(tmp)
+        try:
+            os.link(src, tmp)
+        except OSError:
+            shutil.copyfile(src, tmp)
+        os.replace(tmp, dst)
+
+    def _run_measure(self, manager: Optional[TaskManager], tune_config: TuneConfig, target, args,
+                     gpu_id_default: int = 0) -> None:
+        if tune_config.in_process:
+            target(*args, gpu_id=tune_config.gpu_ids[0] if tune_config.gpu_ids else gpu_id_default)
+        else:
+            manager.add_task(target, args, ident_key="gpu_id")
+
+    # ------------------------------------------------------------------ local stage
+
+    def local_padded_num(self, feat_id: int, occupancy: int, tune_config: TuneConfig) -> int:
+        return self.get_padded_sched_num(len(self.feat_sched_param_candidates[feat_id]),
+                                         tune_config.sm_count * occupancy)
+
+    def compile_local(self, tune_config: TuneConfig) -> None:
+        jobs = []
+        for feat_id in range(self.num_feats):
+            for occupancy in tune_config.occupancies:
+                output_dir, build_dir = self.get_output_build_dir(feat_id, occupancy)
+                if not os.path.exists(f"{build_dir}/librecom.so") or tune_config.recompile:
+                    os.makedirs(build_dir, exist_ok=True)
+                    padded = self.pad_sched_params(self.feat_sched_param_candidates[feat_id],
+                                                   self.local_padded_num(feat_id, occupancy, tune_config))
+                    self.emit_codes(output_dir=output_dir, feat_schedules=padded, occupancy=occupancy,
+                                    inline=tune_config.inline, timing=True, tune=True,
+                                    debug=tune_config.debug, tile_bytes=tune_config.tile_bytes, host=False)
+                    jobs.append((output_dir, build_dir))
+        self._schedule_builds(jobs, tune_config)
+
+    def get_tournament_dir(self, occupancy: int) -> Tuple[str, str]:
+        output_dir = f"{self.basic.codegen_dir}/tournament/o{occupancy}"
+        return output_dir, f"{output_dir}/build"
+
+    def compile_tournament(self, tune_config: TuneConfig) -> None:
+        """One timing build of the whole model per occupancy, holding all candidates."""
+        jobs = []
+        for occupancy in tune_config.occupancies:
+            output_dir, build_dir = self.get_tournament_dir(occupancy)
+            if not os.path.exists(f"{build_dir}/librecom.so") or tune_config.recompile:
+                os.makedirs(build_dir, exist_ok=True)
+                emitter = CodeEmitter(None, feat_candidates=self.feat_sched_param_candidates)
+                emitter.emit(f"{output_dir}/process.hip", occupancy=occupancy, timing=True,
+                             inline=tune_config.inline, tune=True, tile_bytes=tune_config.tile_bytes)
+                emitter.emit_cmake_list(f"{output_dir}/CMakeLists.txt", code_fname="process.hip",
+                                        host_fname=None, subdirs=self.basic.subdirs,
+                                        includes=self.basic.includes, links=self.basic.links,
+                                        debug=tune_config.debug)
+                jobs.append((output_dir, build_dir))
+        self._schedule_builds(jobs, tune_config)
+
+    def tune_in_model(self, tune_config: TuneConfig) -> Dict[int, Dict[int, List[float]]]:
+        self.compile_tournament(tune_config)
+        manager = None if tune_config.in_process else TaskManager(tune_config.gpu_ids)
+        for occupancy in tune_config.occupancies:
+            output_dir, build_dir = self.get_tournament_dir(occupancy)
+            result_log = f"{output_dir}/result.json"
+            if not os.path.exists(result_log) or tune_config.remeasure:
+                args = (occupancy, f"{build_dir}/librecom.so", self.table_shapes, self.data_types,
+                        self.data_npzs, result_log, tune_config.rounds, tune_config.refine_passes,
+                        tune_config.top_k)
+                self._run_measure(manager, tune_config, measure_tournament, args)
+        if manager:
+            manager.join()
+        results: Dict[int, Dict[int, List[float]]] = {feat_id: {} for feat_id in range(self.num_feats)}
+        for occupancy in tune_config.occupancies:
+            output_dir, _ = self.get_tournament_dir(occupancy)
+            with open(f"{output_dir}/result.json") as f:        # absent if the worker failed
+                times = json.load(f)["times"]
+            for feat_id in range(self.num_feats):
+                results[feat_id][occupancy] = times[feat_id]
+        return results
+
+    def tune(self, tune_config: TuneConfig) -> Dict[int, Dict[int, List[float]]]:
+        if tune_config.interference == "model":
+            return self.tune_in_model(tune_config)
+        self.compile_local(tune_config)
+
+        manager = None if tune_config.in_process else TaskManager(tune_config.gpu_ids)
+        for feat_id in range(self.num_feats):
+            for occupancy in tune_config.occupancies:
+                output_dir, build_dir = self.get_output_build_dir(feat_id, occupancy)
+                result_log = f"{output_dir}/result.txt"
+                if not os.path.exists(result_log) or tune_config.remeasure:
+                    args = ((feat_id, occupancy), self.data_npzs[feat_id], self.table_shapes[feat_id],
+                            self.data_types[feat_id], len(self.feat_sched_param_candidates[feat_id]),
+                            self.local_padded_num(feat_id, occupancy, tune_config),
+                            f"{build_dir}/librecom.so", result_log)
+                    self._run_measure(manager, tune_config, measure_single_feat, args)
+        if manager:
+            manager.join()
+
+        results: Dict[int, Dict[int, List[float]]] = {feat_id: {} for feat_id in range(self.num_feats)}
+        for feat_id in range(self.num_feats):
+            for occupancy in tune_config.occupancies:
+                output_dir, build_dir = self.get_output_build_dir(feat_id, occupancy)
+                with open(f"{output_dir}/result.txt") as f:     # absent if the worker failed
+                    results[feat_id][occupancy] = list(map(float, f.read().strip().split(' ')))
+        return results
+
+    # ------------------------------------------------------------------ global stage
+
+    def select_per_occupancy(self, measured_times: Dict[int, Dict[int, List[float]]],
+                             occupancies: Sequence[int]) -> List[List[Tuple[ScheduleBase, NamedTuple]]]:
+        occu_opt_sched_params: List[List[Tuple[ScheduleBase, NamedTuple]]] = [[] for _ in occupancies]
+        for feat_id in range(self.num_feats):
+            for i, occupancy in enumerate(occupancies):
+                opt_idx = int(np.argmin(measured_times[feat_id][occupancy]))
+                occu_opt_sched_params[i].append(self.feat_sched_param_candidates[feat_id][opt_idx])
+        return occu_opt_sched_params
+
+    def solve(self, measured_times: Dict[int, Dict[int, List[float]]],
+              tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
+        occu_opt_sched_params = self.select_per_occupancy(measured_times, tune_config.occupancies)
+        opt_occupancy, opt_sched_params = self.tune_occupancy(occu_opt_sched_params, tune_config)
+        output_dir, build_dir = self.get_output_build_dir(-1, opt_occupancy)
+        optimal = f"{self.basic.codegen_dir}/optimal"
+        shutil.rmtree(optimal, ignore_errors=True)
+        shutil.copytree(output_dir, optimal)
+        with open(f"{optimal}/schedule.json", "w") as f:
+            json.dump({"occupancy": opt_occupancy,
+                       "schedules": CodeEmitter(opt_sched_params).serialize_config()}, f, indent=1)
+        return opt_occupancy, opt_sched_params
+
+    def _build_full(self, output_dir: str, sched_params, occupancy: Optional[int],
+                    tune_config: TuneConfig, fixed_task_block_nums: List[int] = None,
+                    timing: bool = False) -> bool:
+        """Emit a whole-model kernel if its library is missing; True if a build is needed."""
+        build_dir = f"{output_dir}/build"
+        if os.path.exists(f"{build_dir}/librecom.so") and not tune_config.recompile:
+            return False
+        os.makedirs(build_dir, exist_ok=True)
+        self.emit_codes(output_dir=output_dir, feat_schedules=sched_params, occupancy=occupancy,
+                        inline=tune_config.inline, timing=timing, tune=False, debug=tune_config.debug,
+                        fixed_task_block_nums=fixed_task_block_nums, tile_bytes=tune_config.tile_bytes)
+        return True
+
+    def _kernel_time(self, output_dir: str, tune_config: TuneConfig, manager: Optional[TaskManager]) -> None:
+        """Schedule the whole-kernel measurement of the model built in ``output_dir``."""
+        build_dir = f"{output_dir}/build"
+        report_prefix = f"{output_dir}/report"
+        if tune_config.profiler == "rocprofv3":
+            stats = f"{report_prefix}_kernel_stats.csv"
+            if not os.path.exists(stats) or tune_config.remeasure:
+                os_check(f"rm -f {report_prefix}_*.csv")
+                args = (self.table_config_fname, build_dir, self.data_dir, self.basic.sample_batch_nums,
+                        report_prefix)
+                if manager:
+                    manager.add_task(rocprof_profile, args, ident_key="gpu_id")
+                else:
+                    rocprof_profile(*args, gpu_id=tune_config.gpu_ids[0])
+        else:
+            result = f"{report_prefix}.events.txt"
+            if not os.path.exists(result) or tune_config.remeasure:
+                args = (f"{build_dir}/librecom.so", self.table_shapes, self.data_types, self.data_npzs, result)
+                self._run_measure(manager, tune_config, measure_kernel_events, args)
+
+    def _read_kernel_time(self, output_dir: str, tune_config: TuneConfig) -> float:
+        report_prefix = f"{output_dir}/report"
+        if tune_config.profiler == "rocprofv3":
+            return parse_knl_total_time("FusedKnl", f"{report_prefix}_kernel_stats.csv")
+        with open(f"{report_prefix}.events.txt") as f:
+            return float(f.read().strip())
+
+    def _measure_manager(self, tune_config: TuneConfig) -> Optional[TaskManager]:
+        if tune_config.in_process and tune_config.profiler != "rocprofv3":
+            return None
+        if tune_config.profiler == "rocprofv3" and tune_config.in_process:
+            return None      # rocprof_profile spawns its own process; run them one after another
+        return TaskManager(tune_config.gpu_ids[0:1])
+
+    def tune_occupancy(self, occu_opt_sched_params: List[List[Tuple[ScheduleBase, NamedTuple]]],
+                       tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
+        jobs = []
+        for occupancy, sched_params in zip(tune_config.occupancies, occu_opt_sched_params):
+            output_dir, build_dir = self.get_output_build_dir(-1, occupancy)
+            if self._build_full(output_dir, sched_params, occupancy, tune_config):
+                jobs.append((output_dir, build_dir))
+        self._schedule_builds(jobs, tune_config)
+
+        manager = self._measure_manager(tune_config)
+        for occupancy in tune_config.occupancies:
+            output_dir, build_dir = self.get_output_build_dir(-1, occupancy)
+            self._kernel_time(output_dir, tune_config, manager)
+        if manager:
+            manager.join()
+
+        times = []
+        for occupancy in tune_config.occupancies:
+            output_dir, build_dir = self.get_output_build_dir(-1, occupancy)
+            t = self._read_kernel_time(output_dir, tune_config)
+            times.append(t)
+            print(f"occupancy: {occupancy}, t(ns): {t}")
+
+        opt_idx = int(np.argmin(times))
+        return tune_config.occupancies[opt_idx], occu_opt_sched_params[opt_idx]
+
+    # ------------------------------------------------------------------ validation / ablations
+
+    def mutation_validation(self, opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]], opt_occupancy: int,
+                            mut_feat_id: int, tune_config: TuneConfig) -> Tuple[List[float], int]:
+        """Whole-kernel time with feature ``mut_feat_id`` switched to each of its candidates in
+        turn; returns the times and the index of the tuner's own pick."""
+        mutation_dir = f"{self.basic.codegen_dir}/mutation_f{mut_feat_id}"
+        candidates = self.feat_sched_param_candidates[mut_feat_id]
+        opt_idx = -1
+        jobs = []
+        for candidate_id, mut_sched_param in enumerate(candidates):
+            if tuple(mut_sched_param) == tuple(opt_sched_params[mut_feat_id]) or (
+                    type(mut_sched_param[0]) is type(opt_sched_params[mut_feat_id][0])
+                    and mut_sched_param[1] == opt_sched_params[mut_feat_id][1]):
+                opt_idx = candidate_id
+            mut_sched_params = list(opt_sched_params)
+            mut_sched_params[mut_feat_id] = mut_sched_param
+            output_dir = f"{mutation_dir}/m{candidate_id}"
+            if self._build_full(output_dir, mut_sched_params, opt_occupancy, tune_config):
+                jobs.append((output_dir, f"{output_dir}/build"))
+        self._schedule_builds(jobs, tune_config)
+
+        manager = self._measure_manager(tune_config)
+        for candidate_id in range(len(candidates)):
+            self._kernel_time(f"{mutation_dir}/m{candidate_id}", tune_config, manager)
+        if manager:
+            manager.join()
+        times = [self._read_kernel_time(f"{mutation_dir}/m{candidate_id}", tune_config)
+                 for candidate_id in range(len(candidates))]
+        return times, opt_idx
+
+    def tune_naive(self, tune_config: TuneConfig) -> Tuple[List[Tuple[ScheduleBase, NamedTuple]], float]:
+        """Every candidate of every feature measured alone on the GPU (no interference, no
+        occupancy control); the per-feature winners are fused and the whole kernel timed."""
+        def get_output_build_dir(feat_id: int, sched_param_id: int):
+            output_dir = f"{self.basic.codegen_dir}/naive/f{feat_id}/s{sched_param_id}"
+            return output_dir, f"{output_dir}/build"
+
+        jobs = []
+        for feat_id in range(self.num_feats):
+            for sched_param_id, sched_param in enumerate(self.feat_sched_param_candidates[feat_id]):
+                output_dir, build_dir = get_output_build_dir(feat_id, sched_param_id)
+                if not os.path.exists(f"{build_dir}/librecom.so") or tune_config.recompile:
+                    os.makedirs(build_dir, exist_ok=True)
+                    self.emit_codes(output_dir=output_dir, feat_schedules=[sched_param], occupancy=None,
+                                    inline=tune_config.inline, timing=False, tune=False,
+                                    debug=tune_config.debug, tile_bytes=tune_config.tile_bytes, host=False)
+                    jobs.append((output_dir, build_dir))
+        self._schedule_builds(jobs, tune_config)
+
+        manager = None if tune_config.in_process else TaskManager(tune_config.gpu_ids)
+        for feat_id in range(self.num_feats):
+            for sched_param_id in range(len(self.feat_sched_param_candidates[feat_id])):
+                output_dir, build_dir = get_output_build_dir(feat_id, sched_param_id)
+                result_log = f"{output_dir}/result.txt"
+                if not os.path.exists(result_log) or tune_config.remeasure:
+                    args = ((feat_id, sched_param_id), self.data_npzs[feat_id], self.table_shapes[feat_id],
+                            self.data_types[feat_id], f"{build_dir}/librecom.so", result_log)
+                    self._run_measure(manager, tune_config, measure_naive_candidate, args)
+        if manager:
+            manager.join()
+
+        opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]] = []
+        for feat_id in range(self.num_feats):
+            times = []
+            for sched_param_id in range(len(self.feat_sched_param_candidates[feat_id])):
+                output_dir, build_dir = get_output_build_dir(feat_id, sched_param_id)
+                with open(f"{output_dir}/result.txt") as f:
+                    times.append(float(f.read().strip()))
+            opt_sched_params.append(self.feat_sched_param_candidates[feat_id][int(np.argmin(times))])
+
+        output_dir = f"{self.basic.codegen_dir}/naive/optimal"
+        if self._build_full(output_dir, opt_sched_params, None, tune_config):
+            self._schedule_builds([(output_dir, f"{output_dir}/build")], tune_config)
+        manager = self._measure_manager(tune_config)
+        self._kernel_time(output_dir, tune_config, manager)
+        if manager:
+            manager.join()
+        return opt_sched_params, self._read_kernel_time(output_dir, tune_config)
+
+    def tune_fixed_thread_binding(self, opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]], choice: str,
+                                  tune_config: TuneConfig) -> Tuple[List[int], float]:
+        """Ablation: the number of tiles per feature is frozen to the mean / max over the sampled
+        batches of what the run-time binding chose, and baked into the kernel."""
+        assert choice in ["max", "mean"]
+        output_dir = f"{self.basic.codegen_dir}/fixed_thread_binding_{choice}"
+        fixed_blocks_path = f"{output_dir}/task_blocks.txt"
+        if not os.path.exists(fixed_blocks_path) or tune_config.remeasure:
+            os.makedirs(output_dir, exist_ok=True)
+            metas = [s.meta for s, _ in opt_sched_params]
+            measure_task_blocks(self.data_npzs,
+                                [m.row_bytes + INDEX_BYTES for m in metas],
+                                [m.embed_dim * 4 + BAG_FIXED_BYTES for m in metas],
+                                [s.TileGranularity(p) for s, p in opt_sched_params],
+                                tune_config.tile_bytes, fixed_blocks_path)
+
+        task_block_batches: List[List[int]] = []
+        with open(fixed_blocks_path) as f:
+            for line in f.readlines():
+                if line.strip():
+                    task_block_batches.append(list(map(int, line.strip().split(','))))
+
+        if choice == "max":
+            fixed_task_blocks: List[int] = np.max(task_block_batches, axis=0).tolist()
+        else:
+            fixed_task_blocks: List[int] = np.mean(task_block_batches, axis=0, dtype=np.int32).tolist()
+        fixed_task_blocks = [max(1, int(b)) for b in fixed_task_blocks]
+
+        if self._build_full(output_dir, opt_sched_params, None, tune_config,
+                            fixed_task_block_nums=fixed_task_blocks):
+            self._schedule_builds([(output_dir, f"{output_dir}/build")], tune_config)
+        manager = self._measure_manager(tune_config)
+        self._kernel_time(output_dir, tune_config, manager)
+        if manager:
+            manager.join()
+        return fixed_task_blocks, self._read_kernel_time(output_dir, tune_config)

@@ -93,13 +93,43 @@ def test_body_dedup_and_tables():
     assert "__launch_bounds__(BLOCK_THREADS, 4)" in src
     m = re.search(r"c_embed_dim_offsets\[\] = \{\s*([\d,\s]+)\}", src)
     assert [int(v) for v in m.group(1).split(",")] == [0, 32, 64, 128, 160, 192]
-    m = re.search(r"c_process_func_ids\[\] = \{\s*([\d,\s]+)\}", src)
+    m = re.search(r"c_cand_func_ids\[\] = \{\s*([\d,\s]+)\}", src)
     assert [int(v) for v in m.group(1).split(",")] == [0, 0, 2, 0, 4]
+    m = re.search(r"c_cand_begin\[\] = \{\s*([\d,\s]+)\}", src)
+    assert [int(v) for v in m.group(1).split(",")] == [0, 1, 2, 3, 4, 5]
     # bytes per lookup = row bytes + int32 index; per bag = fp32 output slice + one offset
     m = re.search(r"c_lookup_bytes\[\] = \{\s*([\d,\s]+)\}", src)
     assert [int(v) for v in m.group(1).split(",")] == [132, 132, 260, 132, 68]
     m = re.search(r"c_bag_bytes\[\] = \{\s*([\d,\s]+)\}", src)
     assert [int(v) for v in m.group(1).split(",")] == [132, 132, 260, 132, 132]
+
+
+def test_candidate_lists_share_bodies_across_features():
+    """A tuning build carries every candidate of every feature; features with the same dim and
+    element type share all their bodies."""
+    from recflex_amd.schedules import WarpPerSampleSchedule, OneHotSchedule
+    metas = [MetaData(16), MetaData(16), MetaData(32)]
+    cands = []
+    for m in metas:
+        c = []
+        for cls in (OneHotSchedule, WarpPerSampleSchedule):
+            s = cls(m, 256)
+            c.extend((s, p) for p in s.GenParamCandidates())
+        cands.append(c)
+    em = CodeEmitter(None, feat_candidates=cands)
+    assert [len(c) for c in em.feat_candidates] == [len(c) for c in cands]
+    id_map, bodies = em.dedup()
+    n16, n32 = len(cands[0]), len(cands[2])
+    assert len(bodies) <= n16 + n32
+    for i in range(n16):
+        assert id_map[n16 + i] == id_map[i]         # feature 1 reuses feature 0's bodies
+    src = em.emit_kernel(occupancy=4, timing=True)
+    assert f"constexpr int NUM_CANDIDATES = {2 * n16 + n32};" in src
+    m = re.search(r"c_cand_begin\[\] = \{\s*([\d,\s]+)\}", src)
+    assert [int(v) for v in m.group(1).split(",")] == [0, n16, 2 * n16, 2 * n16 + n32]
+    assert em.feat_schedules[0] == cands[0][0]
+    ser = em.serialize_candidates()
+    assert len(ser) == 3 and len(ser[2]) == n32
 
 
 def test_output_vector_width_follows_column_alignment():

@@ -1,0 +1,188 @@
+"""Tuner host logic on the CPU: candidate padding, selection arithmetic against the oracle's
+restatement of tuner.py, resume-by-files, failure of a measurement worker, the compile cache,
+the host restatement of the device binding, and the TaskManager."""
+
+import json
+import multiprocessing as mp
+import os
+
+import numpy as np
+import pytest
+
+from helpers import oracle
+from recflex_amd.code_emitter import MetaData
+from recflex_amd.schedules import SCHEDULE_MAPPING, WarpPerSampleSchedule, OneHotSchedule
+from recflex_amd.tuning import BasicConfig, TuneConfig, Tuner
+from recflex_amd.tuning.tuner import padded_sched_num
+from recflex_amd.tuning.measure import load_batches, save_batches, tiles_per_feature
+
+
+def _tiny_tuner(tmp_path, feats=2, batches=2):
+    rng = np.random.default_rng(5)
+    data = []
+    for f in range(feats):
+        bl = []
+        for _ in range(batches):
+            lens = rng.integers(0, 5, 16)
+            off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            bl.append((rng.integers(0, 100, off[-1]).astype(np.int32), off))
+        data.append(bl)
+    cfg = BasicConfig("", [], "", "", str(tmp_path / "out"), block_threads=256, sample_batch_nums=batches)
+    return Tuner(cfg, SCHEDULE_MAPPING, batches=data, table_shapes=[(100, 16)] * feats,
+                 data_types=["float"] * feats,
+                 schedule_types=[[OneHotSchedule], [WarpPerSampleSchedule]][:feats])
+
+
+def test_padding_matches_reference_rule(tmp_path):
+    t = _tiny_tuner(tmp_path)
+    for n in (1, 5, 24, 152):
+        for m in (1, 108, 256 * 8):
+            assert padded_sched_num(n, m) == oracle.padded_sched_num(n, m)
+            assert t.get_padded_sched_num(n, m) == oracle.padded_sched_num(n, m)
+    cands = t.feat_sched_param_candidates[0]
+    padded = t.pad_sched_params(cands, 2 * len(cands) + 3)
+    assert padded == oracle.pad_sched_params(cands, 2 * len(cands) + 3)
+
+
+def test_selection_is_argmin_per_occupancy(tmp_path):
+    t = _tiny_tuner(tmp_path)
+    n0, n1 = (len(c) for c in t.feat_sched_param_candidates)
+    rng = np.random.default_rng(1)
+    times = {0: {2: rng.random(n0).tolist(), 4: rng.random(n0).tolist()},
+             1: {2: rng.random(n1).tolist(), 4: rng.random(n1).tolist()}}
+    picked = t.select_per_occupancy(times, [2, 4])
+    want = oracle.solve_local(times, [2, 4])
+    for i in range(2):
+        for f in range(2):
+            assert picked[i][f] is t.feat_sched_param_candidates[f][want[i][f]]
+
+
+def test_data_files_round_trip(tmp_path):
+    t = _tiny_tuner(tmp_path)
+    for f in range(2):
+        back = load_batches(t.data_npzs[f])
+        assert len(back) == 2
+        for (i0, o0), (i1, o1) in zip(back, t.batches[f]):
+            assert np.array_equal(i0, i1) and np.array_equal(o0, o1)
+    lines = open(t.table_config_fname).read().split()
+    assert lines == ["100,16,float", "100,16,float"]
+
+
+def test_missing_result_file_raises_like_the_reference(tmp_path):
+    """A measuring worker that fails leaves no result.txt; tune() then raises
+    FileNotFoundError when it collects the results (tuner.py:143-150)."""
+    t = _tiny_tuner(tmp_path)
+    cfg = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=1, in_process=True,
+                     interference="replicate")
+    # pretend the libraries exist so that nothing is compiled; the measurement then fails
+    # (no GPU / not a real library) and is swallowed by the worker
+    for f in range(2):
+        _, build_dir = t.get_output_build_dir(f, 4)
+        os.makedirs(build_dir, exist_ok=True)
+        open(f"{build_dir}/librecom.so", "wb").close()
+    with pytest.raises(FileNotFoundError):
+        t.tune(cfg)
+
+
+def test_resume_uses_existing_results(tmp_path):
+    t = _tiny_tuner(tmp_path)
+    cfg = TuneConfig(occupancies=[2], gpu_ids=[0], sm_count=4, num_processes=1, in_process=True,
+                     interference="replicate")
+    for f in range(2):
+        out, build_dir = t.get_output_build_dir(f, 2)
+        os.makedirs(build_dir, exist_ok=True)
+        open(f"{build_dir}/librecom.so", "wb").close()
+        n = len(t.feat_sched_param_candidates[f])
+        with open(f"{out}/result.txt", "w") as fh:
+            fh.write(" ".join(str(float((k * 7 + f) % n)) for k in range(n)))
+    res = t.tune(cfg)          # neither compiles nor measures
+    assert set(res) == {0, 1} and len(res[0][2]) == len(t.feat_sched_param_candidates[0])
+    assert int(np.argmin(res[0][2])) == 0
+
+
+def test_tournament_results_are_read_back(tmp_path):
+    """Default local stage: one result.json per occupancy under tournament/o{occ}."""
+    t = _tiny_tuner(tmp_path)
+    cfg = TuneConfig(occupancies=[2, 4], gpu_ids=[0], sm_count=4, num_processes=1, in_process=True)
+    counts = [len(c) for c in t.feat_sched_param_candidates]
+    for occ in (2, 4):
+        out, build_dir = t.get_tournament_dir(occ)
+        os.makedirs(build_dir, exist_ok=True)
+        open(f"{build_dir}/librecom.so", "wb").close()
+        times = [[float((k * 3 + occ + f) % n) + 1 for k in range(n)] for f, n in enumerate(counts)]
+        with open(f"{out}/result.json", "w") as fh:
+            json.dump({"times": times, "best": [0, 0]}, fh)
+    res = t.tune(cfg)
+    assert [len(res[f][4]) for f in range(2)] == counts
+    picked = t.select_per_occupancy(res, [2, 4])
+    want = oracle.solve_local(res, [2, 4])
+    assert picked[1][1] is t.feat_sched_param_candidates[1][want[1][1]]
+    os.remove(f"{t.get_tournament_dir(4)[0]}/result.json")
+    with pytest.raises(FileNotFoundError):
+        t.tune(cfg)
+
+
+def test_local_kernel_emission_and_cache_key(tmp_path):
+    t = _tiny_tuner(tmp_path, feats=2)
+    cfg = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=8, num_processes=1)
+    n = len(t.feat_sched_param_candidates[0])
+    assert t.local_padded_num(0, 4, cfg) == oracle.padded_sched_num(n, 32)
+    out, _ = t.get_output_build_dir(0, 4)
+    padded = t.pad_sched_params(t.feat_sched_param_candidates[0], t.local_padded_num(0, 4, cfg))
+    t.emit_codes(out, padded, 4, timing=True, tune=True, host=False)
+    src = open(f"{out}/process.hip").read()
+    assert f"constexpr int NUM_FEATS = {len(padded)};" in src and "TIMING = true" in src
+    assert f"constexpr int NUM_BODIES = {n};" in src
+    key = t._source_key(out)
+    t.emit_codes(out, padded, 4, timing=True, tune=True, host=False)
+    assert t._source_key(out) == key
+    assert not os.path.exists(f"{out}/schedule.json")      # only whole models record theirs
+    t.emit_codes(str(tmp_path / "m"), padded[:3], 4, host=False)
+    cfgs = json.load(open(tmp_path / "m" / "schedule.json"))
+    assert len(cfgs) == 3 and cfgs[0]["schedule"] == "OneHotSchedule"
+
+
+def test_host_binding_restatement():
+    """tiles_per_feature mirrors rfx::bind_tiles: cost / tile_bytes tiles, at least one, at most
+    one per bag; a tile that holds a whole workgroup pass is rounded up to whole passes."""
+    off = np.arange(0, 2049 * 10, 10, dtype=np.int32)          # 2048 bags of 10 lookups
+    # 20480 lookups * 132 B + 2048 * 132 B = 2973696 B -> 46 tiles of 64 KiB wanted
+    tiles = tiles_per_feature([off], [132], [132], [16], 65536)
+    # bags per tile = round_up(ceil(2048 / 46), 16) = 48 -> ceil(2048 / 48) = 43 tiles
+    assert tiles == [43]
+    # a pass of 1024 bags = 1.49 MB > 8 tiles' worth: the tile is not grown to a pass
+    assert tiles_per_feature([off], [132], [132], [1024], 65536) == [46]   # ceil(2048/45)
+    # a pass of 256 bags = 372 KB <= 8 x 64 KiB: whole passes
+    assert tiles_per_feature([off], [132], [132], [256], 65536) == [8]
+    assert tiles_per_feature([off], [132], [132], [1024], 1024) == [2048]  # never more than bags
+    assert tiles_per_feature([off], [132], [132], [16], 1 << 30) == [1]
+    empty = np.zeros(1, dtype=np.int32)
+    assert tiles_per_feature([empty], [132], [132], [16], 65536) == [0]
+
+
+def _sleep_and_record(path, ident=None):
+    import time
+    time.sleep(0.05)
+    with open(path, "a") as f:
+        f.write(f"{ident}\n")
+
+
+def _boom(ident=None):
+    raise RuntimeError("worker failed")
+
+
+def test_task_manager_returns_resources_and_survives_failures(tmp_path):
+    """task_manager.py:27-39: one resource per running task, handed back in `finally`."""
+    from recflex_amd.task_manager import TaskManager
+    if mp.get_start_method(allow_none=True) != "spawn":
+        mp.set_start_method("spawn", force=True)
+    log = str(tmp_path / "log.txt")
+    tm = TaskManager(["gpu0", "gpu1"])
+    for _ in range(5):
+        tm.add_task(_sleep_and_record, (log,), ident_key="ident")
+    tm.add_task(_boom, (), ident_key="ident")
+    tm.join()
+    lines = open(log).read().split()
+    assert len(lines) == 5 and set(lines) <= {"gpu0", "gpu1"}
+    assert tm.resource_queue.qsize() == 2          # both resources are back
+    assert sorted(tm.exit_codes) == [0, 0, 0, 0, 0, 1]
