@@ -35,11 +35,13 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--workload", type=str, default="c3",
                    help="headline configuration (prebuilt model name: c1..c5, c3_tuned)")
-    p.add_argument("--also", type=str, default="c1,c2,c5",
+    p.add_argument("--also", type=str, default="c1,c2,c4,c5",
                    help="comma-separated further configurations reported under 'configs'")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / check leg")
     p.add_argument("--tile-bytes", type=int, default=0)
     p.add_argument("--grid-blocks", type=int, default=0)
+    p.add_argument("--xcd-segments", type=int, default=0,
+                   help="tile walk: 0 = as emitted, -1 = flat, n = n segments per XCD")
     p.add_argument("--copy-calibration", type=int, default=0,
                    help="also launch one plain device-to-device copy of this many bytes (for "
                         "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -118,7 +120,7 @@ def cpu_leg(wl, tables, indices, offsets, gpu_out, max_features: int):
 
 
 def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: int,
-               grid_blocks: int, cpu_features: int) -> dict:
+               grid_blocks: int, cpu_features: int, xcd_segments: int = 0) -> dict:
     import torch
     from recflex_amd import prebuilt
     from recflex_amd.rec_modules import FeatEmbed
@@ -146,7 +148,8 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
     lookups = [len(i) for i in indices]
     alg_bytes = algorithmic_bytes(wl, lookups)
 
-    run = lambda: layer.forward_indices(d_idx, d_off, tile_bytes=tile_bytes, grid_blocks=grid_blocks)
+    run = lambda: layer.forward_indices(d_idx, d_off, tile_bytes=tile_bytes, grid_blocks=grid_blocks,
+                                        xcd_segments=xcd_segments)
     for _ in range(warmup):
         out = run()
     torch.cuda.synchronize()
@@ -165,7 +168,8 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
     outbuf = torch.empty(wl.batch * wl.embed_dim_sum, dtype=torch.float32, device=dev)
     for s, e in zip(starts, ends):
         s.record(stream)
-        layer.forward_indices(d_idx, d_off, tile_bytes=tile_bytes, grid_blocks=grid_blocks, out=outbuf)
+        layer.forward_indices(d_idx, d_off, tile_bytes=tile_bytes, grid_blocks=grid_blocks,
+                              xcd_segments=xcd_segments, out=outbuf)
         e.record(stream)
     torch.cuda.synchronize()
     durs = sorted(s.elapsed_time(e) * 1e3 for s, e in zip(starts, ends))   # us
@@ -216,12 +220,13 @@ def main():
         torch.cuda.empty_cache()
 
     head = run_config(args.workload, args.steps, args.warmup, not args.no_cpu, args.tile_bytes,
-                      args.grid_blocks, args.cpu_features)
+                      args.grid_blocks, args.cpu_features, args.xcd_segments)
     others = {}
     for name in [n for n in args.also.split(",") if n and n != args.workload]:
         try:
             others[name] = run_config(name, args.steps, args.warmup, not args.no_cpu,
-                                      args.tile_bytes, args.grid_blocks, args.cpu_features)
+                                      args.tile_bytes, args.grid_blocks, args.cpu_features,
+                                      args.xcd_segments)
         except Exception as exc:  # a configuration that does not fit must not hide the headline
             others[name] = {"error": f"{type(exc).__name__}: {exc}"}
 

@@ -63,10 +63,18 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--workload", type=str, help="built-in synthetic configuration (c1..c5)")
     parser.add_argument("--workload_batches", type=int, default=2)
     parser.add_argument("--compile_only", action="store_true", default=False)
+    parser.add_argument("--launch_only", action="store_true", default=False,
+                        help="skip the local stage: default schedules, swept over occupancy and the "
+                             "launch parameters of the run-time binding")
     parser.add_argument("--occupancies", type=str, help="comma-separated workgroups per CU to try")
     parser.add_argument("--sample_batch_nums", type=int, default=128)
     parser.add_argument("--profiler", type=str, default="rocprofv3", choices=["rocprofv3", "events"])
     parser.add_argument("--tile_bytes", type=int, default=0)
+    parser.add_argument("--tile_bytes_candidates", type=str,
+                        help="comma-separated traffic-per-tile values swept in the global stage")
+    parser.add_argument("--xcd_segments_candidates", type=str,
+                        help="comma-separated tile-walk settings swept in the global stage "
+                             "(-1 = flat, n > 0 = n segments per XCD)")
     parser.add_argument("--interference", type=str, default="model", choices=["model", "replicate"],
                         help="local stage: candidates timed inside the whole model, or per feature "
                              "against copies of themselves (the reference's scheme)")
@@ -132,6 +140,10 @@ def create_tune_config(args: argparse.Namespace) -> TuneConfig:
     kwargs = {}
     if args.tile_bytes:
         kwargs["tile_bytes"] = args.tile_bytes
+    if args.xcd_segments_candidates:
+        kwargs["xcd_segments_candidates"] = [int(v) for v in args.xcd_segments_candidates.split(",")]
+    if args.tile_bytes_candidates:
+        kwargs["tile_bytes_candidates"] = [int(v) for v in args.tile_bytes_candidates.split(",")]
     return TuneConfig(occupancies=occupancies, gpu_ids=gpu_ids, sm_count=sm_count,
                       num_processes=args.num_processes, recompile=args.recompile,
                       remeasure=args.remeasure, inline=not args.noinline, debug=args.debug,
@@ -149,6 +161,11 @@ def main():
         else:
             tuner.compile_local(tune_config)
         print(f"local-stage kernels built under {tuner.basic.codegen_dir}")
+        return
+
+    if args.launch_only:
+        occupancy, sched_params = tuner.solve_launch_only(tune_config)
+        print(occupancy, tuner.opt_tile_bytes, tuner.opt_xcd_segments)
         return
 
     if not args.naive:

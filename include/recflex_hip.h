@@ -53,7 +53,8 @@ typedef struct recom_info {
   int32_t tile_bytes;     /* default memory traffic per tile used by the run-time binding */
   int32_t static_binding; /* 1 if the tile count per feature was fixed at emit time */
   int32_t num_candidates; /* schedules compiled in; == num_features unless a tuning build */
-  int32_t reserved[6];
+  int32_t xcd_segments;   /* default of recom_process_args.xcd_segments (0 = flat tile walk) */
+  int32_t reserved[5];
 } recom_info;
 
 #define RECOM_ABI_VERSION 1
@@ -119,12 +120,18 @@ typedef struct recom_process_args {
   int32_t tile_bytes;
   /* persistent grid size; 0 = recom_get_max_concurrent_blocks() */
   int32_t grid_blocks;
+  /* L2 locality of the tile walk: > 0 cuts the (feature-ordered) tile space into 8 * xcd_segments
+   * equal segments and gives segment s to the workgroups of XCD s % 8, so that the rows a
+   * feature's bags share are cached by one or two of the eight L2s instead of all; 0 = the
+   * emitted default; < 0 = flat walk (tile t to workgroup t % grid) */
+  int32_t xcd_segments;
   /* tuning builds: device int32[F], the candidate schedule each feature runs in this launch
    * (clamped to the feature's candidate count); NULL = candidate 0 everywhere */
   const int32_t *d_schedule_choice;
   /* timing builds only: device uint64[F], the kernel ADDS each feature's workgroup-ticks
    * (s_memtime) to it; caller zeroes it.  Replaces the per-block clock() array
-   * (RecFlex/code_emitter/codegen.py:301-316,388-401).  Must be NULL otherwise. */
+   * (RecFlex/code_emitter/codegen.py:301-316,388-401).  NULL runs a timing build untimed;
+   * must be NULL for other builds. */
   unsigned long long *d_times;
   /* hipStream_t to launch on (NULL = the null stream) */
   void *stream;

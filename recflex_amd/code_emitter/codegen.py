@@ -32,6 +32,11 @@ XCD_COUNT = 8
 # per-bag traffic that does not depend on the bag length, besides the output slice: one offset
 BAG_FIXED_BYTES = 4
 INDEX_BYTES = 4
+# The binding sizes tiles by cost = lookups * (row bytes + index + this) + bags * (output + offset):
+# a lookup costs time that does not shrink with the row (address arithmetic, a memory round
+# trip), expressed here as extra bytes so that tiles of narrow-row features do not run longer
+# than tiles of wide-row features.
+LOOKUP_OVERHEAD_BYTES = 0
 
 
 def _c_array(ctype: str, name: str, values: List[int], per_line: int = 16) -> str:
@@ -134,8 +139,11 @@ class CodeEmitter:
 
     def emit_kernel(self, occupancy: int = None, inline: bool = True, timing: bool = False,
                     timing_branch: bool = False, fixed_task_block_nums: List[int] = None,
-                    tile_bytes: int = None, xcd_aware: bool = False) -> str:
+                    tile_bytes: int = None, xcd_aware: bool = False,
+                    lookup_overhead_bytes: int = None, xcd_segments: int = 8) -> str:
         num_feats = len(self.feat_schedules)
+        if lookup_overhead_bytes is None:
+            lookup_overhead_bytes = LOOKUP_OVERHEAD_BYTES
         assert num_feats > 0, "cannot emit a fused kernel for zero features"
         vars_ = ScheduleVars()
         id_map, body_ids = self.dedup()
@@ -150,7 +158,8 @@ constexpr int OCCUPANCY = {occupancy if occupancy else 0};
 constexpr int TILE_BYTES = {tile_bytes if tile_bytes else DEFAULT_TILE_BYTES};
 constexpr int NUM_BODIES = {len(body_ids)};
 constexpr int NUM_CANDIDATES = {len(flat)};
-constexpr int XCDS = {XCD_COUNT if xcd_aware else 1};
+constexpr int XCDS = {XCD_COUNT};
+constexpr int XCD_SEGMENTS = {xcd_segments if xcd_aware else 0};
 constexpr bool TIMING = {"true" if timing else "false"};
 constexpr bool STATIC_BINDING = {"true" if fixed_task_block_nums else "false"};
 
@@ -181,7 +190,8 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
         tables += _c_array("int", "c_cand_gran", [s.TileGranularity(p) for s, p in flat])
         tables += _c_array("int", "c_embed_dim_offsets", embed_dim_offsets)
         tables += _c_array("int", "c_lookup_bytes",
-                           [s.meta.row_bytes + INDEX_BYTES for s, _ in self.feat_schedules])
+                           [s.meta.row_bytes + INDEX_BYTES + lookup_overhead_bytes
+                            for s, _ in self.feat_schedules])
         tables += _c_array("int", "c_bag_bytes",
                            [s.meta.embed_dim * 4 + BAG_FIXED_BYTES for s, _ in self.feat_schedules])
         if fixed_task_block_nums:
@@ -189,14 +199,34 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
             tables += _c_array("int", "c_fixed_task_block_nums",
                                [max(1, int(n)) for n in fixed_task_block_nums])
 
+        # Timing builds: each workgroup adds the ticks of its tiles per feature in LDS and flushes
+        # them to d_times once, when it has run out of tiles (an atomic per tile would sit in front
+        # of the next tile's loads).  With d_times == nullptr a timing build runs untimed.
         timing_begin = '''
-    __syncthreads();
-    const unsigned long long t_begin = __builtin_amdgcn_s_memtime();
+    unsigned long long t_begin = 0;
+    if (d_times) {
+      __syncthreads();
+      t_begin = __builtin_amdgcn_s_memtime();
+    }
 ''' if timing else ''
         timing_end = '''
+    if (d_times) {
+      __syncthreads();
+      if (threadIdx.x == 0)
+        s_ticks[feat_idx] += static_cast<unsigned int>(__builtin_amdgcn_s_memtime() - t_begin);
+    }
+''' if timing else ''
+        timing_init = f'''
+  __shared__ unsigned int s_ticks[NUM_FEATS];
+  if (d_times)
+    for (int f = threadIdx.x; f < NUM_FEATS; f += {vars_.BLOCK_THREADS}) s_ticks[f] = 0;
+''' if timing else ''
+        timing_flush = f'''
+  if (d_times) {{
     __syncthreads();
-    if (threadIdx.x == 0)
-      atomicAdd(&d_times[feat_idx], __builtin_amdgcn_s_memtime() - t_begin);
+    for (int f = threadIdx.x; f < NUM_FEATS; f += {vars_.BLOCK_THREADS})
+      if (s_ticks[f]) atomicAdd(&d_times[f], static_cast<unsigned long long>(s_ticks[f]));
+  }}
 ''' if timing else ''
 
         call_args = (f"table, indices, offsets, d_output, embed_dim_offset, "
@@ -214,30 +244,40 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     const char *__restrict__ d_arg_buffers,
     const int64_t *__restrict__ d_arg_buffer_offsets,
     float *__restrict__ d_output,
-    const int batch, const int tile_bytes,
+    const int batch, const int tile_bytes, const int xcd_segments,
     const int *__restrict__ d_schedule_choice,
     unsigned long long *__restrict__ d_times) {{
   __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;
 
   __shared__ KnlTempStorage s;
-
+{timing_init}
   const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
   const int total_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}>(
       s_bind, io, tile_bytes, c_lookup_bytes, c_bag_bytes, c_cand_begin, c_cand_gran,
       d_schedule_choice, {"c_fixed_task_block_nums" if fixed_task_block_nums else "nullptr"});
 
-  // Tiles are ordered by feature.  Workgroup i runs on XCD i % XCDS, so the workgroups of one
-  // XCD walk one contiguous 1/XCDS of the tile space: the rows a feature's bags share stay in
-  // that XCD's L2 instead of being fetched into all of them.
-  int tile_first = blockIdx.x, tile_last = total_tiles, tile_step = gridDim.x;
-  if (XCDS > 1 && gridDim.x % XCDS == 0) {{
-    const int chunk = (total_tiles + XCDS - 1) / XCDS;
-    const int xcd = blockIdx.x % XCDS;
-    tile_first = xcd * chunk + blockIdx.x / XCDS;
-    tile_last = min(total_tiles, (xcd + 1) * chunk);
-    tile_step = gridDim.x / XCDS;
+  // Tiles are ordered by feature.  Workgroup i runs on XCD i % XCDS.  With xcd_segments > 0 the
+  // tile space is cut into XCDS * xcd_segments equal segments and segment s belongs to XCD
+  // s % XCDS: a feature's tiles
+  // -- and the table rows its bags share -- stay in the L2 of one or two XCDs instead of being
+  // fetched into all of them, while every XCD still gets a sample of all kinds of features.
+  int walk_first = blockIdx.x, walk_last = total_tiles, walk_step = gridDim.x;
+  int xcd = 0, seg_len = 1;
+  const bool by_xcd = xcd_segments > 0 && gridDim.x % XCDS == 0;
+  if (by_xcd) {{
+    seg_len = (total_tiles + XCDS * xcd_segments - 1) / (XCDS * xcd_segments);
+    xcd = blockIdx.x % XCDS;
+    walk_first = blockIdx.x / XCDS;
+    walk_last = seg_len * xcd_segments;
+    walk_step = gridDim.x / XCDS;
   }}
-  for (int tile = tile_first; tile < tile_last; tile += tile_step) {{
+  for (int walk = walk_first; walk < walk_last; walk += walk_step) {{
+    int tile = walk;
+    if (by_xcd) {{
+      const int seg = walk / seg_len;
+      tile = (seg * XCDS + xcd) * seg_len + (walk - seg * seg_len);
+      if (tile >= total_tiles) continue;
+    }}
 {timing_begin if timing and timing_branch else ''}
     const int feat_idx = __builtin_amdgcn_readfirstlane(rfx::find_feature<NUM_FEATS>(s_bind, tile));
     const int bags_per_tile = s_bind.bags_per_tile[feat_idx];
@@ -253,7 +293,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     }}
 {timing_end}
   }}
-}}
+{timing_flush}}}
 
 '''
         return consts + temp_storage_decl + functions + "\n" + tables + kernel
@@ -264,8 +304,9 @@ extern "C" int recom_process(const recom_process_args *a) {
   if (!a || !a->d_embed_table_ptrs || !a->d_output || a->batch < 0 ||
       (!a->d_io_ptrs && (!a->d_arg_buffers || !a->d_arg_buffer_offsets)))
     return static_cast<int>(hipErrorInvalidValue);
-  if (TIMING != (a->d_times != nullptr)) return static_cast<int>(hipErrorInvalidValue);
-  if (a->tile_bytes < 0 || a->grid_blocks < 0) return static_cast<int>(hipErrorInvalidValue);
+  if (!TIMING && a->d_times) return static_cast<int>(hipErrorInvalidValue);
+  if (a->tile_bytes < 0 || a->grid_blocks < 0 || a->xcd_segments > 4096)
+    return static_cast<int>(hipErrorInvalidValue);
   if (a->batch == 0) return static_cast<int>(hipSuccess);
 
   const rfx::LaunchState *st = nullptr;
@@ -274,12 +315,15 @@ extern "C" int recom_process(const recom_process_args *a) {
   const int grid = a->grid_blocks > 0 ? a->grid_blocks : st->cus * st->occupancy;
   if (grid <= 0) return static_cast<int>(hipErrorInvalidConfiguration);
   const int tile_bytes = a->tile_bytes > 0 ? a->tile_bytes : TILE_BYTES;
+  const int xcd_segments = a->xcd_segments > 0 ? a->xcd_segments
+                                               : (a->xcd_segments < 0 ? 0 : XCD_SEGMENTS);
 
   hipLaunchKernelGGL(FusedKnl, dim3(grid), dim3(BLOCK_THREADS), st->dyn_lds,
                      static_cast<hipStream_t>(a->stream),
                      a->d_embed_table_ptrs, a->d_io_ptrs,
                      static_cast<const char *>(a->d_arg_buffers), a->d_arg_buffer_offsets,
-                     a->d_output, a->batch, tile_bytes, a->d_schedule_choice, a->d_times);
+                     a->d_output, a->batch, tile_bytes, xcd_segments, a->d_schedule_choice,
+                     a->d_times);
   return static_cast<int>(hipGetLastError());
 }
 '''
@@ -328,6 +372,7 @@ extern "C" int recom_get_info(recom_info *out) {
   out->tile_bytes = TILE_BYTES;
   out->static_binding = STATIC_BINDING ? 1 : 0;
   out->num_candidates = NUM_CANDIDATES;
+  out->xcd_segments = XCD_SEGMENTS;
   return 0;
 }
 
@@ -376,7 +421,8 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
     def emit(self, ofname: str, occupancy: int = None, inline: bool = True,
              tune: bool = False, timing: bool = False, timing_branch: bool = False,
              fixed_task_block_nums: List[int] = None, tile_bytes: int = None,
-             xcd_aware: bool = False) -> None:
+             xcd_aware: bool = False, lookup_overhead_bytes: int = None,
+             xcd_segments: int = 8) -> None:
         """Write the device source.  ``occupancy`` = workgroups per CU the kernel is built and
         launched for (``__launch_bounds__`` budget, persistent grid size, and a dynamic-LDS pad
         that keeps further workgroups off the CU); ``tune`` is accepted for signature
@@ -386,7 +432,9 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
         code += self.emit_kernel(timing=timing, timing_branch=timing_branch,
                                  occupancy=occupancy, inline=inline,
                                  fixed_task_block_nums=fixed_task_block_nums,
-                                 tile_bytes=tile_bytes, xcd_aware=xcd_aware)
+                                 tile_bytes=tile_bytes, xcd_aware=xcd_aware,
+                                 lookup_overhead_bytes=lookup_overhead_bytes,
+                                 xcd_segments=xcd_segments)
         code += self.emit_process_func(timing=timing, occupancy=occupancy)
         code += self.emit_get_concurrent_blocks_func(occupancy=occupancy)
         code += self.emit_process_ops()

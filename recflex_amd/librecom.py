@@ -25,7 +25,8 @@ class RecomInfo(ctypes.Structure):
         ("tile_bytes", ctypes.c_int32),
         ("static_binding", ctypes.c_int32),
         ("num_candidates", ctypes.c_int32),
-        ("reserved", ctypes.c_int32 * 6),
+        ("xcd_segments", ctypes.c_int32),
+        ("reserved", ctypes.c_int32 * 5),
     ]
 
 
@@ -48,6 +49,7 @@ class RecomProcessArgs(ctypes.Structure):
         ("batch", ctypes.c_int32),
         ("tile_bytes", ctypes.c_int32),
         ("grid_blocks", ctypes.c_int32),
+        ("xcd_segments", ctypes.c_int32),
         ("d_schedule_choice", ctypes.c_void_p),
         ("d_times", ctypes.c_void_p),
         ("stream", ctypes.c_void_p),
@@ -134,12 +136,13 @@ class RecomLib:
 
     def process(self, table_ptrs: int, output: int, batch: int, *, io_ptrs: int = 0,
                 arg_buffers: int = 0, arg_buffer_offsets: int = 0, tile_bytes: int = 0,
-                grid_blocks: int = 0, schedule_choice: int = 0, times: int = 0,
-                stream: int = 0) -> None:
+                grid_blocks: int = 0, xcd_segments: int = 0, schedule_choice: int = 0,
+                times: int = 0, stream: int = 0) -> None:
         """All pointer arguments are raw device addresses (``tensor.data_ptr()``)."""
         args = RecomProcessArgs(table_ptrs or None, io_ptrs or None, arg_buffers or None,
                                 arg_buffer_offsets or None, output or None, batch, tile_bytes,
-                                grid_blocks, schedule_choice or None, times or None, stream or None)
+                                grid_blocks, xcd_segments, schedule_choice or None, times or None,
+                                stream or None)
         rc = self.lib.recom_process(ctypes.byref(args))
         if rc != 0:
             raise RecomError("recom_process", rc)

@@ -5,7 +5,9 @@ GPU machines only load what is already built here; ``ensure_built`` compiles a m
 its library is missing.  Names:
 
 ``c1`` .. ``c5``     the five benchmark configurations at full size, default (untuned) schedules
-``c3_tuned``       C3 with the schedules in ``recflex_amd/tuned/c3_schedule.json`` if present
+``cN_tuned``       CN with the schedules, occupancy and launch parameters recorded in
+                   ``recflex_amd/tuned/cN_schedule.json`` (written by ``examples/tune.py``); the
+                   default build if that file is absent
 ``c3_xcd``         C3 with the XCD-aware tile walk switched on (for comparison)
 ``c2s`` .. ``c5s``   shrunken C2..C5 (fewer rows / features / samples) that a CPU checker can follow
 ``variants``       one feature per (element type, dim, schedule candidate) over a spread of the
@@ -71,7 +73,12 @@ def _tuned(wl: Workload, fname: str) -> ModelSpec:
     fs = load_feat_schedules(tmp, BLOCK_THREADS)
     os.remove(tmp)
     assert len(fs) == wl.num_features
-    return ModelSpec(wl, fs, occupancy)
+    kwargs = {}
+    if isinstance(doc, dict) and doc.get("tile_bytes"):
+        kwargs["tile_bytes"] = doc["tile_bytes"]
+    if isinstance(doc, dict) and doc.get("xcd_segments", 0) > 0:
+        kwargs.update(xcd_aware=True, xcd_segments=doc["xcd_segments"])
+    return ModelSpec(wl, fs, occupancy, kwargs)
 
 
 def _variants() -> ModelSpec:
@@ -116,7 +123,10 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c3": lambda: _default(make_workload("C3")),
     "c4": lambda: _default(make_workload("C4")),
     "c5": lambda: _default(make_workload("C5")),
+    "c2_tuned": lambda: _tuned(make_workload("C2"), "c2_schedule.json"),
     "c3_tuned": lambda: _tuned(make_workload("C3"), "c3_schedule.json"),
+    "c4_tuned": lambda: _tuned(make_workload("C4"), "c4_schedule.json"),
+    "c5_tuned": lambda: _tuned(make_workload("C5"), "c5_schedule.json"),
     "c3_xcd": lambda: _default(make_workload("C3"), xcd_aware=True),
     "c2s": lambda: _default(make_workload("C2", batch=512, max_rows=200_000)),
     "c3s": lambda: _default(make_workload("C3", batch=192, max_rows=60_000)),

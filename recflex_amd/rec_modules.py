@@ -152,7 +152,7 @@ class FeatEmbed(nn.Module):
 
     def _launch(self, batch: int, timing: bool, timing_schedules: Optional[int], tile_bytes: int,
                 grid_blocks: int, schedule_choice: torch.Tensor = None, out: torch.Tensor = None,
-                **inputs):
+                xcd_segments: int = 0, **inputs):
         if out is not None:
             if out.dtype != torch.float32 or out.numel() != batch * self.output_units \
                     or not out.is_contiguous() or out.device.type != "cuda":
@@ -162,10 +162,10 @@ class FeatEmbed(nn.Module):
         else:
             output = torch.empty([batch * self.output_units], dtype=torch.float32, device=self.device)
         times = None
-        if self.lib.info.timing:
+        if timing:
+            if not self.lib.info.timing:
+                raise RuntimeError("timing=True needs a library emitted with timing=True")
             times = torch.zeros([self.lib.num_features], dtype=torch.int64, device=self.device)
-        elif timing:
-            raise RuntimeError("timing=True needs a library emitted with timing=True")
         if schedule_choice is not None:
             if schedule_choice.dtype != torch.int32 or schedule_choice.numel() != len(self.embed_tables) \
                     or schedule_choice.device.type != "cuda":
@@ -173,7 +173,7 @@ class FeatEmbed(nn.Module):
             inputs["schedule_choice"] = schedule_choice.data_ptr()
         stream = torch.cuda.current_stream(self.device).cuda_stream
         self.lib.process(self.embed_table_ptrs.data_ptr(), output.data_ptr(), batch,
-                         tile_bytes=tile_bytes, grid_blocks=grid_blocks,
+                         tile_bytes=tile_bytes, grid_blocks=grid_blocks, xcd_segments=xcd_segments,
                          times=times.data_ptr() if times is not None else 0, stream=stream, **inputs)
         if timing:
             n = len(self.embed_tables)
@@ -206,7 +206,7 @@ class FeatEmbed(nn.Module):
     def forward_indices(self, indices: Sequence[torch.Tensor], offsets: Sequence[torch.Tensor],
                         timing: bool = False, timing_schedules: int = None, tile_bytes: int = 0,
                         grid_blocks: int = 0, schedule_choice: torch.Tensor = None,
-                        out: torch.Tensor = None):
+                        out: torch.Tensor = None, xcd_segments: int = 0):
         """Per-feature int32 device tensors ``indices[f]`` (``[L_f]``) and ``offsets[f]``
         (``[batch + 1]``, exclusive prefix sums, ``offsets[f][0] == 0``) -> ``[batch, sum(dim)]``
         fp32 (with ``timing=True``: ``(output, task_times)``).  ``out``: write into this
@@ -215,21 +215,22 @@ class FeatEmbed(nn.Module):
         if len(indices) != n or len(offsets) != n:
             raise ValueError(f"expected {n} index and offset tensors")
         batch = offsets[0].numel() - 1
-        for f in range(n):
-            for name, t in (("indices", indices[f]), ("offsets", offsets[f])):
-                if t.dtype != torch.int32 or not t.is_contiguous() or t.device.type != "cuda":
-                    raise TypeError(f"{name}[{f}] must be a contiguous int32 device tensor")
-            if offsets[f].numel() != batch + 1:
-                raise ValueError("all features must share one batch size")
-        key = tuple(t.data_ptr() for t in indices) + tuple(t.data_ptr() for t in offsets)
+        key = tuple(t.data_ptr() for t in indices) + tuple(t.data_ptr() for t in offsets) + (batch,)
         if key != self._io_cache_key:
+            # new input tensors: validate them and upload their addresses
+            for f in range(n):
+                for name, t in (("indices", indices[f]), ("offsets", offsets[f])):
+                    if t.dtype != torch.int32 or not t.is_contiguous() or t.device.type != "cuda":
+                        raise TypeError(f"{name}[{f}] must be a contiguous int32 device tensor")
+                if offsets[f].numel() != batch + 1:
+                    raise ValueError("all features must share one batch size")
             flat = [0] * (2 * n)
             flat[0::2] = [t.data_ptr() for t in indices]
             flat[1::2] = [t.data_ptr() for t in offsets]
             self._io_ptrs = torch.tensor(flat, dtype=torch.int64, device=self.device)
             self._io_cache_key = key
         res = self._launch(batch, timing, timing_schedules, tile_bytes, grid_blocks,
-                           schedule_choice=schedule_choice, out=out,
+                           schedule_choice=schedule_choice, out=out, xcd_segments=xcd_segments,
                            io_ptrs=self._io_ptrs.data_ptr())
         if timing:
             return res[0].view(batch, self.output_units), res[1]

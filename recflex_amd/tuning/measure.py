@@ -59,12 +59,15 @@ def save_batches(data_npz: str, batches: Sequence[Tuple[np.ndarray, np.ndarray]]
 
 def make_table(table_shape: Tuple[int, int], data_type: str, device, ones: bool = True):
     """Table of the right storage type; ``ones`` as in the reference's tuning runs
-    (``measure.py:41``), else N(0, 1)."""
+    (``measure.py:41``), else N(0, 0.01)."""
     import torch
     from recflex_amd.quant import quantize_rowwise_int8
+    from recflex_amd.workloads import FeatureSpec, gen_table
     rows, dim = table_shape
-    w = torch.ones(rows, dim, dtype=torch.float32, device=device) if ones else \
-        torch.randn(rows, dim, dtype=torch.float32, device=device)
+    if not ones:       # built chunk by chunk: no fp32 copy of a large fp16 / int8 table
+        return gen_table(FeatureSpec(rows, dim, data_type, 1.0, True, 0.0, 0.0), seed=rows + dim,
+                         device=device)
+    w = torch.ones(rows, dim, dtype=torch.float32, device=device)
     if data_type == "half":
         return w.half()
     if data_type == "int8":
@@ -77,6 +80,25 @@ def _write_atomically(path: str, text: str) -> None:
     with open(tmp, "w") as f:
         f.write(text)
     os.replace(tmp, path)
+
+
+def _timed_launches(launch, reps: int, burst: int = 4) -> float:
+    """Median over ``reps`` of the time per launch in ns.  Each sample brackets ``burst``
+    back-to-back launches with one event pair, after one launch that keeps the GPU busy while the
+    host queues them, so that the host's launch overhead is not part of the measurement."""
+    import torch
+    samples = []
+    for _ in range(reps):
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        launch()
+        start.record()
+        for _ in range(burst):
+            launch()
+        end.record()
+        end.synchronize()
+        samples.append(start.elapsed_time(end) * 1e6 / burst)
+    return sorted(samples)[len(samples) // 2]
 
 
 def measure_single_feat(ident: Tuple[int, int], data_npz: str, table_shape: Tuple[int, int],
@@ -115,6 +137,7 @@ def measure_tournament(ident: int, librecom_path: str, table_shapes: Sequence[Tu
                        data_types: Sequence[str], data_npzs: Sequence[str], output_path: str,
                        rounds: int = 3, refine_passes: int = 3, top_k: int = 8,
                        probe_fraction: float = 0.2, probes_per_candidate: int = 3, seed: int = 0,
+                       climb_passes: int = 1, start_choices: Sequence[Sequence[int]] = (),
                        gpu_id: int = None) -> Optional[List[List[float]]]:
     """Local stage inside the real model: the library holds every candidate of every feature
     and each launch runs one candidate per feature (``d_schedule_choice``), so a candidate is
@@ -125,8 +148,17 @@ def measure_tournament(ident: int, librecom_path: str, table_shapes: Sequence[Tu
     tile time.  Refinement, ``refine_passes`` times: every feature runs its current best except a
     random ``probe_fraction`` of the features, each of which tries one of its ``top_k``
     candidates; the scores measured against this near-final background replace the exploration
-    scores of those candidates and the best is re-elected.  Writes
-    ``{"times": [[score per candidate] per feature], "best": [...]}`` as JSON."""
+    scores of those candidates and the best is re-elected.
+
+    Whole-kernel climb, ``climb_passes`` times: tile times are a zero-sum measure once the kernel
+    is bound by memory bandwidth (a schedule that keeps more loads in flight finishes its own
+    tiles sooner by slowing the others down), so the elected mix -- or any of ``start_choices``
+    (e.g. the untuned default) that runs faster -- is then improved against the kernel's own
+    duration: feature by feature, heaviest first, each of the feature's ``top_k`` candidates is
+    swapped in and kept if the whole launch gets faster.  The kept candidates get the lowest
+    score of their feature, so that an argmin over the scores reproduces the final mix.
+
+    Writes ``{"times": [[score per candidate] per feature], "best": [...], "kernel_ns": t}``."""
     print(f"Tournament, Occ {ident}, GPU {gpu_id}", flush=True)
     try:
         _pin_gpu(gpu_id)
@@ -193,9 +225,49 @@ def measure_tournament(ident: int, librecom_path: str, table_shapes: Sequence[Tu
                 # candidate that was measured against the incumbent mix
                 score[f] = np.where(seen, refined, np.maximum(score[f], worst_seen))
                 best[f] = int(np.argmin(score[f]))
+        # ---- whole-kernel climb
+        outs = [layer.forward_indices(d_idx, d_off) for d_idx, d_off in device_batches]
+
+        def kernel_ns(choice: np.ndarray, reps: int = 3) -> float:
+            d_choice = torch.from_numpy(choice.astype(np.int32)).to(dev)
+            total = 0.0
+            for (d_idx, d_off), out in zip(device_batches, outs):
+                total += _timed_launches(
+                    lambda: layer.forward_indices(d_idx, d_off, out=out, schedule_choice=d_choice), reps)
+            return total
+
+        best_ns = None
+        if climb_passes > 0:
+            for _ in range(10):
+                kernel_ns(best, reps=1)                      # clocks up
+            best_ns = kernel_ns(best, reps=5)
+            for start in start_choices:
+                cand = np.array([min(max(int(c), 0), n - 1) for c, n in zip(start, counts)])
+                t = kernel_ns(cand, reps=5)
+                print(f"[tournament {ident}] start mix {t:.0f} ns vs elected {best_ns:.0f} ns", flush=True)
+                if t < best_ns:
+                    best, best_ns = cand, t
+            share = launch(best)
+            order = np.argsort(-share)
+            for _ in range(climb_passes):
+                for f in order:
+                    for c in np.argsort(score[f])[:min(top_k, counts[f])]:
+                        if c == best[f]:
+                            continue
+                        trial = best.copy()
+                        trial[f] = c
+                        t = kernel_ns(trial)
+                        if t < best_ns * 0.995:
+                            t = kernel_ns(trial, reps=5)     # confirm before keeping
+                            if t < best_ns * 0.995:
+                                best, best_ns = trial, t
+            for f in range(num_feats):
+                score[f][best[f]] = min(score[f].min(), score[f][best[f]]) * 0.999
+            print(f"[tournament {ident}] kernel after climb {best_ns:.0f} ns", flush=True)
         torch.cuda.synchronize()
         result = [sc.tolist() for sc in score]
-        _write_atomically(output_path, json.dumps({"times": result, "best": best.tolist()}))
+        _write_atomically(output_path, json.dumps({"times": result, "best": [int(b) for b in best],
+                                                   "kernel_ns": best_ns}))
         return result
     except Exception as e:
         print(f"[tournament {ident}] Exception {type(e).__name__}: {e}", flush=True)
@@ -220,14 +292,8 @@ def measure_naive_candidate(ident: Tuple[int, int], data_npz: str, table_shape: 
         for idx, off in load_batches(data_npz):
             d_idx = [torch.from_numpy(idx).to(dev)]
             d_off = [torch.from_numpy(off).to(dev)]
-            layer.forward_indices(d_idx, d_off)          # warm-up (first launch sets the grid up)
-            start = torch.cuda.Event(enable_timing=True)
-            end = torch.cuda.Event(enable_timing=True)
-            start.record()
-            layer.forward_indices(d_idx, d_off)
-            end.record()
-            end.synchronize()
-            accum_ms += start.elapsed_time(end)
+            out = layer.forward_indices(d_idx, d_off)    # warm-up (first launch sets the grid up)
+            accum_ms += _timed_launches(lambda: layer.forward_indices(d_idx, d_off, out=out), 3) / 1e6
         _write_atomically(output_path, str(accum_ms))
         return accum_ms
     except Exception as e:
@@ -247,7 +313,8 @@ def _run_script_args(table_config_fname: str, build_dir: str, data_dir: str,
 
 
 def rocprof_profile(table_config_fname: str, build_dir: str, data_dir: str, sample_batch_nums: int,
-                    report_prefix: str, spec_feat_id: int = None, gpu_id: int = None) -> None:
+                    report_prefix: str, spec_feat_id: int = None, tile_bytes: int = 0,
+                    xcd_segments: int = 0, gpu_id: int = None) -> None:
     """Leaves ``{report_prefix}_kernel_stats.csv`` (rocprofv3 ``--kernel-trace --stats``)."""
     if gpu_id is None:
         raise Exception("No valid GPU provided!")
@@ -256,7 +323,8 @@ def rocprof_profile(table_config_fname: str, build_dir: str, data_dir: str, samp
     name = os.path.basename(report_prefix)
     cmd = [rocprof, "--kernel-trace", "--stats", "--output-format", "csv", "-d", out_dir, "-o", name,
            "--"] + _run_script_args(table_config_fname, build_dir, data_dir, sample_batch_nums,
-                                    spec_feat_id)
+                                    spec_feat_id) + ["--tile_bytes", str(tile_bytes),
+                                                    "--xcd_segments", str(xcd_segments)]
     env = dict(os.environ)
     env["HIP_VISIBLE_DEVICES"] = str(gpu_id)
     env.setdefault("TMPDIR", "/tmp")
@@ -270,7 +338,8 @@ nsys_profile = rocprof_profile
 
 def measure_kernel_events(librecom_path: str, table_shapes: Sequence[Tuple[int, int]],
                           data_types: Sequence[str], data_npzs: Sequence[str], output_path: str,
-                          repeats: int = 20, warmup: int = 10, gpu_id: int = None) -> Optional[float]:
+                          tile_bytes: int = 0, xcd_segments: int = 0, repeats: int = 7, warmup: int = 10,
+                          gpu_id: int = None) -> Optional[float]:
     """Total FusedKnl time in ns over all batches (median of ``repeats`` launches per batch),
     measured with events on the launch stream; written to ``output_path``."""
     try:
@@ -288,17 +357,11 @@ def measure_kernel_events(librecom_path: str, table_shapes: Sequence[Tuple[int, 
             d_off = [torch.from_numpy(b[k][1]).to(dev) for b in per_feat]
             out = layer.forward_indices(d_idx, d_off)       # its buffer is reused below
             for _ in range(warmup):                         # let the clocks settle
-                layer.forward_indices(d_idx, d_off, out=out)
-            times = []
-            for _ in range(repeats):
-                start = torch.cuda.Event(enable_timing=True)
-                end = torch.cuda.Event(enable_timing=True)
-                start.record()
-                layer.forward_indices(d_idx, d_off, out=out)
-                end.record()
-                end.synchronize()
-                times.append(start.elapsed_time(end) * 1e6)
-            total_ns += sorted(times)[len(times) // 2]
+                layer.forward_indices(d_idx, d_off, out=out, tile_bytes=tile_bytes,
+                                      xcd_segments=xcd_segments)
+            total_ns += _timed_launches(
+                lambda: layer.forward_indices(d_idx, d_off, out=out, tile_bytes=tile_bytes,
+                                              xcd_segments=xcd_segments), repeats)
         _write_atomically(output_path, str(total_ns))
         return total_ns
     except Exception as e:

@@ -21,6 +21,8 @@ if __name__ == "__main__":
     parser.add_argument("--sample_batch_nums", type=int, required=True)
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--repeats", type=int, default=1)
+    parser.add_argument("--tile_bytes", type=int, default=0)
+    parser.add_argument("--xcd_segments", type=int, default=0)
     args = parser.parse_args()
 
     import torch
@@ -58,6 +60,7 @@ if __name__ == "__main__":
     prof.start()
     for _ in range(args.repeats):
         for d_idx, d_off in device_batches:
-            output = layer.forward_indices(d_idx, d_off)
+            output = layer.forward_indices(d_idx, d_off, tile_bytes=args.tile_bytes,
+                                           xcd_segments=args.xcd_segments)
     torch.cuda.synchronize()
     prof.stop()

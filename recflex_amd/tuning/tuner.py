@@ -79,6 +79,17 @@ class TuneConfig(NamedTuple):
     rounds: int = 3
     refine_passes: int = 3
     top_k: int = 8
+    # passes of the whole-kernel climb that follows the tile-time tournament (0 = none)
+    climb_passes: int = 1
+    # global stage: traffic-per-tile values of the run-time binding to try for every occupancy
+    # (a launch parameter, no rebuild); empty = only tile_bytes
+    tile_bytes_candidates: List[int] = []
+    # global stage: L2-locality settings of the tile walk to try (launch parameter
+    # xcd_segments; -1 = flat walk); empty = only the emitted default
+    xcd_segments_candidates: List[int] = []
+    # global stage: also time the untuned default schedules at every occupancy and keep them
+    # if they win (tile times measured feature by feature do not always add up to kernel time)
+    include_default: bool = True
 
 
 def padded_sched_num(orig_num: int, max_concurrent_blocks: int) -> int:
@@ -196,13 +207,14 @@ class Tuner:
     def emit_codes(self, output_dir: str, feat_schedules: List[Tuple[ScheduleBase, NamedTuple]],
                    occupancy: int, inline: bool = True, timing: bool = False, tune: bool = False,
                    fixed_task_block_nums: List[int] = None, debug: bool = False,
-                   tile_bytes: int = None, host: bool = True) -> None:
+                   tile_bytes: int = None, host: bool = True, xcd_segments: int = 0) -> None:
         os.makedirs(output_dir, exist_ok=True)
         emitter = CodeEmitter(feat_schedules)
         if host:
             emitter.emit_host(f"{output_dir}/preprocess.cpp", fixed_task_block_nums=fixed_task_block_nums)
         emitter.emit(f"{output_dir}/process.hip", occupancy=occupancy, timing=timing, inline=inline, tune=tune,
-                     fixed_task_block_nums=fixed_task_block_nums, tile_bytes=tile_bytes)
+                     fixed_task_block_nums=fixed_task_block_nums, tile_bytes=tile_bytes,
+                     xcd_aware=xcd_segments > 0, xcd_segments=max(xcd_segments, 1))
         emitter.emit_cmake_list(f"{output_dir}/CMakeLists.txt", code_fname="process.hip",
                                 host_fname="preprocess.cpp" if host else None,
                                 subdirs=self.basic.subdirs, includes=self.basic.includes, links=self.basic.links,
@@ -310,6 +322,30 @@ class Tuner:
                 jobs.append((output_dir, build_dir))
         self._schedule_builds(jobs, tune_config)
 
+    def default_choices(self) -> List[List[int]]:
+        """Index, in every feature's candidate list, of the schedule ``default_schedule`` would
+        pick from the mean bag length of the sampled batches (nearest candidate of the same
+        template if the exact parameters are not in the list): a known-good mix the climb may
+        start from."""
+        from recflex_amd.schedules import default_schedule
+        choice = []
+        for feat_id, cands in enumerate(self.feat_sched_param_candidates):
+            lens = [len(i) / max(1, len(o) - 1) for i, o in self.batches[feat_id]]
+            sched, params = default_schedule(self.metas[feat_id], float(np.mean(lens)),
+                                             self.basic.block_threads)
+            body = sched.EmitScheduleBody(params)
+            pick, best_d = 0, None
+            for k, (s, p) in enumerate(cands):
+                if s.EmitScheduleBody(p) == body:
+                    pick, best_d = k, -1
+                    break
+                if type(s) is type(sched):
+                    d = sum(abs(a - b) for a, b in zip(p, params))
+                    if best_d is None or d < best_d:
+                        pick, best_d = k, d
+            choice.append(pick)
+        return [choice]
+
     def tune_in_model(self, tune_config: TuneConfig) -> Dict[int, Dict[int, List[float]]]:
         self.compile_tournament(tune_config)
         manager = None if tune_config.in_process else TaskManager(tune_config.gpu_ids)
@@ -319,7 +355,8 @@ class Tuner:
             if not os.path.exists(result_log) or tune_config.remeasure:
                 args = (occupancy, f"{build_dir}/librecom.so", self.table_shapes, self.data_types,
                         self.data_npzs, result_log, tune_config.rounds, tune_config.refine_passes,
-                        tune_config.top_k)
+                        tune_config.top_k, 0.2, 3, 0, tune_config.climb_passes,
+                        self.default_choices())
                 self._run_measure(manager, tune_config, measure_tournament, args)
         if manager:
             manager.join()
@@ -374,14 +411,35 @@ class Tuner:
               tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
         occu_opt_sched_params = self.select_per_occupancy(measured_times, tune_config.occupancies)
         opt_occupancy, opt_sched_params = self.tune_occupancy(occu_opt_sched_params, tune_config)
-        output_dir, build_dir = self.get_output_build_dir(-1, opt_occupancy)
+        output_dir = self.opt_output_dir
         optimal = f"{self.basic.codegen_dir}/optimal"
         shutil.rmtree(optimal, ignore_errors=True)
         shutil.copytree(output_dir, optimal)
+        tile_bytes = getattr(self, "opt_tile_bytes", tune_config.tile_bytes)
+        xcd_segments = getattr(self, "opt_xcd_segments", 0)
+        if tile_bytes != tune_config.tile_bytes or xcd_segments:
+            # make the winning launch parameters the defaults of the optimal library
+            self.emit_codes(output_dir=optimal, feat_schedules=opt_sched_params, occupancy=opt_occupancy,
+                            inline=tune_config.inline, debug=tune_config.debug, tile_bytes=tile_bytes,
+                            xcd_segments=max(xcd_segments, 0))
+            shutil.rmtree(f"{optimal}/build", ignore_errors=True)   # the copied CMake cache names another dir
+            compile_build(f"{optimal}/build")
         with open(f"{optimal}/schedule.json", "w") as f:
-            json.dump({"occupancy": opt_occupancy,
+            json.dump({"occupancy": opt_occupancy, "tile_bytes": tile_bytes,
+                       "xcd_segments": max(xcd_segments, 0),
                        "schedules": CodeEmitter(opt_sched_params).serialize_config()}, f, indent=1)
         return opt_occupancy, opt_sched_params
+
+    def solve_launch_only(self, tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
+        """Global stage alone: the default schedule of every feature, swept over occupancy, traffic
+        per tile and tile walk.  Needs no tuning build; ends like ``solve`` with ``optimal/``."""
+        default_mix = [self.feat_sched_param_candidates[f][k]
+                       for f, k in enumerate(self.default_choices()[0])]
+        cfg = tune_config._replace(include_default=False)
+        results = {f: {occ: [0.0 if c is default_mix[f] else 1.0
+                             for c in self.feat_sched_param_candidates[f]]
+                       for occ in cfg.occupancies} for f in range(self.num_feats)}
+        return self.solve(results, cfg)
 
     def _build_full(self, output_dir: str, sched_params, occupancy: Optional[int],
                     tune_config: TuneConfig, fixed_task_block_nums: List[int] = None,
@@ -396,16 +454,23 @@ class Tuner:
                         fixed_task_block_nums=fixed_task_block_nums, tile_bytes=tune_config.tile_bytes)
         return True
 
-    def _kernel_time(self, output_dir: str, tune_config: TuneConfig, manager: Optional[TaskManager]) -> None:
-        """Schedule the whole-kernel measurement of the model built in ``output_dir``."""
+    @staticmethod
+    def _report_prefix(output_dir: str, tile_bytes: int, xcd_segments: int) -> str:
+        return (f"{output_dir}/report" + (f".t{tile_bytes}" if tile_bytes else "")
+                + (f".x{xcd_segments}" if xcd_segments else ""))
+
+    def _kernel_time(self, output_dir: str, tune_config: TuneConfig, manager: Optional[TaskManager],
+                     tile_bytes: int = 0, xcd_segments: int = 0) -> None:
+        """Schedule the whole-kernel measurement of the model built in ``output_dir``
+        (0 = the traffic per tile / tile walk the library was emitted with)."""
         build_dir = f"{output_dir}/build"
-        report_prefix = f"{output_dir}/report"
+        report_prefix = self._report_prefix(output_dir, tile_bytes, xcd_segments)
         if tune_config.profiler == "rocprofv3":
             stats = f"{report_prefix}_kernel_stats.csv"
             if not os.path.exists(stats) or tune_config.remeasure:
                 os_check(f"rm -f {report_prefix}_*.csv")
                 args = (self.table_config_fname, build_dir, self.data_dir, self.basic.sample_batch_nums,
-                        report_prefix)
+                        report_prefix, None, tile_bytes, xcd_segments)
                 if manager:
                     manager.add_task(rocprof_profile, args, ident_key="gpu_id")
                 else:
@@ -413,11 +478,13 @@ class Tuner:
         else:
             result = f"{report_prefix}.events.txt"
             if not os.path.exists(result) or tune_config.remeasure:
-                args = (f"{build_dir}/librecom.so", self.table_shapes, self.data_types, self.data_npzs, result)
+                args = (f"{build_dir}/librecom.so", self.table_shapes, self.data_types, self.data_npzs,
+                        result, tile_bytes, xcd_segments)
                 self._run_measure(manager, tune_config, measure_kernel_events, args)
 
-    def _read_kernel_time(self, output_dir: str, tune_config: TuneConfig) -> float:
-        report_prefix = f"{output_dir}/report"
+    def _read_kernel_time(self, output_dir: str, tune_config: TuneConfig, tile_bytes: int = 0,
+                          xcd_segments: int = 0) -> float:
+        report_prefix = self._report_prefix(output_dir, tile_bytes, xcd_segments)
         if tune_config.profiler == "rocprofv3":
             return parse_knl_total_time("FusedKnl", f"{report_prefix}_kernel_stats.csv")
         with open(f"{report_prefix}.events.txt") as f:
@@ -432,29 +499,47 @@ class Tuner:
 
     def tune_occupancy(self, occu_opt_sched_params: List[List[Tuple[ScheduleBase, NamedTuple]]],
                        tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
-        jobs = []
+        # contenders: (directory, occupancy, schedules)
+        contenders = []
         for occupancy, sched_params in zip(tune_config.occupancies, occu_opt_sched_params):
-            output_dir, build_dir = self.get_output_build_dir(-1, occupancy)
+            contenders.append((self.get_output_build_dir(-1, occupancy)[0], occupancy, sched_params))
+        if tune_config.include_default:
+            default_mix = [self.feat_sched_param_candidates[f][k]
+                           for f, k in enumerate(self.default_choices()[0])]
+            for occupancy in tune_config.occupancies:
+                contenders.append((f"{self.basic.codegen_dir}/default/o{occupancy}", occupancy, default_mix))
+
+        jobs = []
+        for output_dir, occupancy, sched_params in contenders:
             if self._build_full(output_dir, sched_params, occupancy, tune_config):
-                jobs.append((output_dir, build_dir))
+                jobs.append((output_dir, f"{output_dir}/build"))
         self._schedule_builds(jobs, tune_config)
 
+        launch_opts = [(tb, xs) for tb in (list(tune_config.tile_bytes_candidates) or [0])
+                       for xs in (list(tune_config.xcd_segments_candidates) or [0])]
         manager = self._measure_manager(tune_config)
-        for occupancy in tune_config.occupancies:
-            output_dir, build_dir = self.get_output_build_dir(-1, occupancy)
-            self._kernel_time(output_dir, tune_config, manager)
+        for output_dir, occupancy, _ in contenders:
+            for tile_bytes, xcd_segments in launch_opts:
+                self._kernel_time(output_dir, tune_config, manager, tile_bytes, xcd_segments)
         if manager:
             manager.join()
 
-        times = []
-        for occupancy in tune_config.occupancies:
-            output_dir, build_dir = self.get_output_build_dir(-1, occupancy)
-            t = self._read_kernel_time(output_dir, tune_config)
-            times.append(t)
-            print(f"occupancy: {occupancy}, t(ns): {t}")
+        times, best_opts = [], []
+        for output_dir, occupancy, _ in contenders:
+            per_opt = [self._read_kernel_time(output_dir, tune_config, tb, xs) for tb, xs in launch_opts]
+            k = int(np.argmin(per_opt))
+            times.append(per_opt[k])
+            best_opts.append(launch_opts[k])
+            kind = "default" if "/default/o" in output_dir else "tuned"
+            print(f"occupancy: {occupancy} ({kind}), t(ns): {per_opt[k]}"
+                  + (f", (tile_bytes, xcd_segments): {launch_opts[k]} (of "
+                     f"{ {o: round(t) for o, t in zip(launch_opts, per_opt)} })" if len(launch_opts) > 1 else ""))
 
         opt_idx = int(np.argmin(times))
-        return tune_config.occupancies[opt_idx], occu_opt_sched_params[opt_idx]
+        self.opt_tile_bytes = best_opts[opt_idx][0] or tune_config.tile_bytes
+        self.opt_xcd_segments = best_opts[opt_idx][1]
+        self.opt_output_dir, opt_occupancy, opt_sched_params = contenders[opt_idx]
+        return opt_occupancy, opt_sched_params
 
     # ------------------------------------------------------------------ validation / ablations
 

@@ -53,10 +53,10 @@ def test_host_library_exports_every_host_symbol():
 
 
 def test_ctypes_structs_match_header_layout():
-    # recom_info: 10 named int32 + 6 reserved; recom_process_args: 5 pointers, 3 int32 (+pad),
+    # recom_info: 11 named int32 + 5 reserved; recom_process_args: 5 pointers, 4 int32,
     # 3 pointers on LP64
     assert ctypes.sizeof(RecomInfo) == 16 * 4
-    assert ctypes.sizeof(RecomProcessArgs) == 5 * 8 + 3 * 4 + 4 + 3 * 8
+    assert ctypes.sizeof(RecomProcessArgs) == 5 * 8 + 4 * 4 + 3 * 8
     assert RecomProcessArgs.batch.offset == 40 and RecomProcessArgs.d_schedule_choice.offset == 56
     assert RecomProcessArgs.d_times.offset == 64
     src = open(HEADER).read()

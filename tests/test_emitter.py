@@ -143,7 +143,8 @@ def test_emit_variants_and_file_update(tmp_path):
     f = tmp_path / "process.hip"
     em.emit(str(f), occupancy=2, timing=True)
     src = f.read_text()
-    assert "TIMING = true" in src and "s_memtime" in src and "atomicAdd(&d_times[feat_idx]" in src
+    assert "TIMING = true" in src and "s_memtime" in src and "s_ticks[feat_idx] +=" in src
+    assert "atomicAdd(&d_times[f]" in src
     assert 'extern "C" int recom_process' in src and 'extern "C" int recom_get_info' in src
     mtime = f.stat().st_mtime_ns
     em.emit(str(f), occupancy=2, timing=True)            # unchanged -> not rewritten
