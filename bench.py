@@ -25,6 +25,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0   # MI355X, HBM3E, published
 METRIC = "fused-kernel us + achieved HBM GB/s (% of MI355X peak) per model config"
 
+# HBM bytes per launch (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, rocprofv3 --pmc, scale factors
+# from a 1 GiB copy in the same runs) of the tuned models, as recorded in
+# profiles/FusedKnl_c3_c2_c5.md; a live run cannot read these counters itself.
+MEASURED_TRAFFIC_BYTES = {"c3_tuned": 548.5e6, "c2_tuned": 44.5e6, "c5_tuned": 7621e6}
+
 TOL = {"float": (1e-5, 1e-6), "half": (1e-3, 1e-6), "int8": (1e-3, 1e-6)}
 
 
@@ -254,7 +259,7 @@ def main():
         "pct_of_peak": head["pct_of_peak"],
         "roofline": {"bound": "hbm", "achieved": head["achieved_gbps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": head["achieved_gbps"] / HBM_PEAK_GBPS,
-                     "traffic": None, "kernel": "FusedKnl",
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(head["model"]), "kernel": "FusedKnl",
                      "algorithmic_bytes_per_launch": head["algorithmic_bytes"]},
     }
     if "cpu_baseline" in head:
