@@ -193,31 +193,34 @@ def gen_inputs(wl: Workload) -> Tuple[List[np.ndarray], List[np.ndarray]]:
     return indices, offsets
 
 
-def _gen_integer_table(spec: FeatureSpec, g, device):
+def _integer_rows(spec: FeatureSpec, g, device, n: int):
+    """``n`` rows of small integers (int8: integer codes, scale in {1/4, 1/2, 1, 2}, integer
+    bias), for which every fp32 sum of a few thousand rows is exact in any order."""
     import torch
     from .quant import int8_row_stride
     if spec.data_type != "int8":
-        w = torch.randint(-8, 9, (spec.rows, spec.dim), generator=g, device=device)
+        w = torch.randint(-8, 9, (n, spec.dim), generator=g, device=device, dtype=torch.int32)
         return w.to(torch.float32 if spec.data_type == "float" else torch.float16)
-    out = torch.zeros(spec.rows, int8_row_stride(spec.dim), dtype=torch.uint8, device=device)
-    out[:, :spec.dim] = torch.randint(0, 256, (spec.rows, spec.dim), generator=g, device=device).to(torch.uint8)
+    out = torch.zeros(n, int8_row_stride(spec.dim), dtype=torch.uint8, device=device)
+    out[:, :spec.dim] = torch.randint(0, 256, (n, spec.dim), generator=g, device=device,
+                                      dtype=torch.int32).to(torch.uint8)
     scale = torch.tensor([0.25, 0.5, 1.0, 2.0], device=device)[
-        torch.randint(0, 4, (spec.rows,), generator=g, device=device)]
-    bias = torch.randint(-8, 9, (spec.rows,), generator=g, device=device).float()
+        torch.randint(0, 4, (n,), generator=g, device=device)]
+    bias = torch.randint(-8, 9, (n,), generator=g, device=device).float()
     sb = torch.stack([scale, bias], dim=1).half().contiguous()
-    out[:, spec.dim:spec.dim + 4] = sb.view(torch.uint8).view(spec.rows, 4)
+    out[:, spec.dim:spec.dim + 4] = sb.view(torch.uint8).view(n, 4)
     return out
 
 
 def gen_table(spec: FeatureSpec, seed: int, device, chunk_rows: int = 1 << 21,
               table_values: str = "normal"):
-    """Device table of one feature: N(0, 0.01) fp32, rounded to fp16, or row-wise int8."""
+    """Device table of one feature: N(0, 0.01) fp32, rounded to fp16, or row-wise int8
+    (``table_values="integer"``: small integers instead).  Filled in chunks of rows so that the
+    temporaries stay small beside tables that nearly fill the device."""
     import torch
     from .quant import int8_row_stride, quantize_rowwise_int8
     g = torch.Generator(device=device)
     g.manual_seed(seed)
-    if table_values == "integer":
-        return _gen_integer_table(spec, g, device)
     if spec.data_type == "float":
         out = torch.empty(spec.rows, spec.dim, dtype=torch.float32, device=device)
     elif spec.data_type == "half":
@@ -226,6 +229,9 @@ def gen_table(spec: FeatureSpec, seed: int, device, chunk_rows: int = 1 << 21,
         out = torch.empty(spec.rows, int8_row_stride(spec.dim), dtype=torch.uint8, device=device)
     for r0 in range(0, spec.rows, chunk_rows):
         r1 = min(spec.rows, r0 + chunk_rows)
+        if table_values == "integer":
+            out[r0:r1] = _integer_rows(spec, g, device, r1 - r0)
+            continue
         w = torch.randn(r1 - r0, spec.dim, dtype=torch.float32, device=device, generator=g) * TABLE_STD
         if spec.data_type == "int8":
             out[r0:r1] = quantize_rowwise_int8(w)

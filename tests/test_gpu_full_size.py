@@ -1,0 +1,122 @@
+"""GPU parity at the full sizes of the benchmark configurations, through the C ABI of the
+prebuilt (tuned) libraries.
+
+Where the CPU oracle finishes in seconds (C2, C3) the whole output is compared with it.  For all
+of C3, C4 and C5 -- up to 260 GB of tables and 2.7e8 lookups -- size-independent properties are
+checked instead, on integer-valued tables for which every fp32 sum is exact whatever its order:
+
+* row checksums: for every feature and bag, the sum over the feature's output columns equals the
+  sum over the bag's lookups of the looked-up rows' own sums;
+* column checksums: for every feature and column, the sum over all bags equals the sum over all
+  lookups of that column of the looked-up rows;
+
+both computed with stock torch reductions on the device (no kernel of this package, no oracle),
+and both exact, so the comparison is on equality.  A misplaced column, a dropped or doubled
+lookup, a wrong bag boundary or a wrong row address changes at least one of them.
+"""
+
+import gc
+
+import numpy as np
+import pytest
+
+from helpers import check_against_oracle, oracle_output, require_lib
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(name: str, table_values: str = None):
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    wl = prebuilt.model_spec(name).workload
+    if table_values:
+        wl = wl._replace(table_values=table_values)
+    dev = torch.device("cuda", 0)
+    print(f"[case] model={name} F={wl.num_features} B={wl.batch} tables={wl.table_bytes() / 1e9:.1f} GB "
+          f"values={wl.table_values}", flush=True)
+    gc.collect()
+    torch.cuda.empty_cache()        # hand back what earlier tests' tables left in torch's cache
+    free, _ = torch.cuda.mem_get_info(dev)
+    assert wl.table_bytes() < 0.95 * free, f"{name}: tables do not fit ({free / 1e9:.0f} GB free)"
+    tables = gen_tables(wl, dev)
+    indices, offsets = gen_inputs(wl)
+    d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+    d_off = [torch.from_numpy(o).to(dev) for o in offsets]
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib(name))
+    return wl, dev, tables, indices, offsets, d_idx, d_off, layer
+
+
+@pytest.mark.parametrize("name", ["c2_tuned", "c3_tuned"])
+def test_full_size_matches_oracle(name):
+    import torch
+    wl, dev, tables, indices, offsets, d_idx, d_off, layer = _setup(name)
+    out = layer.forward_indices(d_idx, d_off)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    want = oracle_output(wl, [t.cpu().numpy() for t in tables], indices, offsets)
+    failures = check_against_oracle(wl, got, want)
+    assert not failures, f"{len(failures)} features out of tolerance, first {failures[:3]}"
+    if name.startswith("c2"):       # bags of one lookup: a row copy
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def _decoded(rows, spec):
+    """fp32 values of table rows (torch restatement of the three row formats)."""
+    import torch
+    if spec.data_type != "int8":
+        return rows.float()
+    codes = rows[:, :spec.dim].float()
+    sb = rows[:, spec.dim:spec.dim + 4].contiguous().view(torch.float16).float()
+    return codes * sb[:, 0:1] + sb[:, 1:2]
+
+
+@pytest.mark.parametrize("name", ["c3_tuned", "c5_tuned", "c4_tuned"])
+def test_full_size_checksums(name):
+    import torch
+    wl, dev, tables, indices, offsets, d_idx, d_off, layer = _setup(name, table_values="integer")
+    out = layer.forward_indices(d_idx, d_off)
+    torch.cuda.synchronize()
+    assert out.shape == (wl.batch, wl.embed_dim_sum)
+
+    chunk = 1 << 20
+    col = 0
+    bad = []
+    for f, spec in enumerate(wl.features):
+        slab = out[:, col:col + spec.dim]
+        col += spec.dim
+        idx = d_idx[f].long()
+        lens = (d_off[f][1:] - d_off[f][:-1]).long()
+        assert int(d_off[f][-1]) == idx.numel()
+        bag_of = torch.repeat_interleave(torch.arange(wl.batch, device=dev), lens)
+        want_rows = torch.zeros(wl.batch, dtype=torch.float64, device=dev)
+        want_cols = torch.zeros(spec.dim, dtype=torch.float64, device=dev)
+        for p0 in range(0, idx.numel(), chunk):
+            vals = _decoded(tables[f].index_select(0, idx[p0:p0 + chunk]), spec).double()
+            want_cols += vals.sum(0)
+            want_rows.index_add_(0, bag_of[p0:p0 + chunk], vals.sum(1))
+        assert idx.numel() == 0 or float(want_cols.abs().sum()) > 0      # the check is not vacuous
+        got_rows = slab.sum(1, dtype=torch.float64)
+        got_cols = slab.sum(0, dtype=torch.float64)
+        if not (torch.equal(got_rows, want_rows) and torch.equal(got_cols, want_cols)):
+            bad.append((f, spec, int((got_rows != want_rows).sum()), int((got_cols != want_cols).sum())))
+        if f % 50 == 0:
+            print(f"  feature {f} checked", flush=True)
+    assert not bad, f"{len(bad)} features with wrong checksums, first {bad[:3]}"
+
+
+def test_launch_parameters_do_not_change_a_bit():
+    """Tile size, grid size and the tile walk decide which workgroup sums a bag, never the order
+    of the sum inside it: the full-size C3 output must be identical bit for bit."""
+    import torch
+    wl, dev, tables, indices, offsets, d_idx, d_off, layer = _setup("c3_tuned")
+    ref = layer.forward_indices(d_idx, d_off).clone()
+    for kwargs in ({"tile_bytes": 8192}, {"tile_bytes": 1 << 20, "xcd_segments": -1},
+                   {"grid_blocks": 300, "xcd_segments": 3}, {"xcd_segments": 64},
+                   {"grid_blocks": 8, "xcd_segments": 1}):
+        print(f"  launch {kwargs}", flush=True)
+        out = layer.forward_indices(d_idx, d_off, **kwargs)
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int32), ref.view(torch.int32)), kwargs

@@ -9,7 +9,8 @@ from helpers import check_against_oracle, oracle_output, require_lib
 pytestmark = pytest.mark.gpu
 
 
-def _run_model(name: str, form: str = "pointers", tile_bytes: int = 0, grid_blocks: int = 0):
+def _run_model(name: str, form: str = "pointers", tile_bytes: int = 0, grid_blocks: int = 0,
+               xcd_segments: int = 0):
     import torch
     from recflex_amd import prebuilt
     from recflex_amd.rec_modules import FeatEmbed
@@ -20,14 +21,15 @@ def _run_model(name: str, form: str = "pointers", tile_bytes: int = 0, grid_bloc
     wl = spec.workload
     dev = torch.device("cuda", 0)
     print(f"[case] model={name} form={form} F={wl.num_features} B={wl.batch} "
-          f"tile_bytes={tile_bytes} grid={grid_blocks}", flush=True)
+          f"tile_bytes={tile_bytes} grid={grid_blocks} xcd_segments={xcd_segments}", flush=True)
     tables = gen_tables(wl, dev)
     indices, offsets = gen_inputs(wl)
     layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib(name))
     if form == "pointers":
         d_idx = [torch.from_numpy(i).to(dev) for i in indices]
         d_off = [torch.from_numpy(o).to(dev) for o in offsets]
-        out = layer.forward_indices(d_idx, d_off, tile_bytes=tile_bytes, grid_blocks=grid_blocks)
+        out = layer.forward_indices(d_idx, d_off, tile_bytes=tile_bytes, grid_blocks=grid_blocks,
+                                    xcd_segments=xcd_segments)
     else:
         packed, byte_offsets = RecomHost().pack(offsets, indices)
         out = layer(torch.from_numpy(packed).to(dev), torch.from_numpy(byte_offsets).to(dev),
@@ -57,10 +59,13 @@ def test_packed_buffer_form(name):
     _assert_parity(*_run_model(name, form="packed"))
 
 
-@pytest.mark.parametrize("tile_bytes,grid", [(4096, 0), (1 << 20, 0), (0, 1), (0, 7), (16384, 3)])
-def test_binding_is_result_invariant(tile_bytes, grid):
-    """Any tile size / grid size must give the same pooled output (only the binding changes)."""
-    _assert_parity(*_run_model("c3s", tile_bytes=tile_bytes, grid_blocks=grid))
+@pytest.mark.parametrize("tile_bytes,grid,xcd", [(4096, 0, 0), (1 << 20, 0, 0), (0, 1, 0), (0, 7, 0),
+                                                 (16384, 3, 0), (0, 0, -1), (0, 0, 1), (4096, 0, 16),
+                                                 (0, 5, 2), (0, 1024, 1000)])
+def test_binding_is_result_invariant(tile_bytes, grid, xcd):
+    """Any tile size / grid size / tile walk must give the same pooled output (only the binding
+    changes); grids that are not a multiple of the 8 XCDs and more segments than tiles included."""
+    _assert_parity(*_run_model("c3s", tile_bytes=tile_bytes, grid_blocks=grid, xcd_segments=xcd))
 
 
 @pytest.mark.parametrize("name", ["variants", "edge"])
