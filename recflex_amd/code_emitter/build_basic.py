@@ -33,7 +33,15 @@ class BasicBuilder:
             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
             "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
         ]
+        # e.g. RECFLEX_HIP_EXTRA_FLAGS="-DRFX_PREFETCH_GROUPS=0" for an experiment
+        self.hip_flags += os.environ.get("RECFLEX_HIP_EXTRA_FLAGS", "").split()
         self.host_flags: List[str] = ["-std=c++17", "-shared", "-fPIC", "-Wall"]
+
+    def device_headers(self) -> List[str]:
+        """The headers every emitted ``process.hip`` is built from."""
+        names = sorted(n for n in os.listdir(self.include) if n.endswith(".h"))
+        return [os.path.join(self.include, n) for n in names] + \
+               [os.path.join(self.abi_include, "recflex_hip.h")]
 
     def host_lib_path(self, dirname: str = "build") -> str:
         return os.path.join(self.csrc_dir, dirname, "librecflex_host.so")

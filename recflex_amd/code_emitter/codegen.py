@@ -514,13 +514,15 @@ extern "C" int recom_host_preprocess_feat(
         host_link_flags = " ".join(host_links)
         opt = "-g -O0" if debug else "-O3"
         add_subdirs = '\n'.join(f"add_subdirectory({subdir})" for subdir in subdirs)
+        # the device side is header-only: a change of a schedule template rebuilds the library
+        device_headers = " ".join(basic.device_headers())
 
         recom = f'''
 add_custom_command(
   OUTPUT ${{CMAKE_BINARY_DIR}}/librecom.so
   COMMAND {basic.hipcc} {" ".join(basic.hip_flags)} {opt} {inc_flags}
           ${{CMAKE_SOURCE_DIR}}/{code_fname} {link_flags} -o ${{CMAKE_BINARY_DIR}}/librecom.so
-  DEPENDS ${{CMAKE_SOURCE_DIR}}/{code_fname}
+  DEPENDS ${{CMAKE_SOURCE_DIR}}/{code_fname} {device_headers}
   VERBATIM)
 add_custom_target(recom ALL DEPENDS ${{CMAKE_BINARY_DIR}}/librecom.so)
 ''' if code_fname else ''

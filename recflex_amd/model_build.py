@@ -38,6 +38,8 @@ def build_model(output_dir: str, feat_schedules: FeatSchedules, rebuild: bool = 
     lib = f"{output_dir}/build/librecom.so"
     if rebuild or not os.path.exists(lib):
         emit_model(output_dir, feat_schedules, **emit_kwargs)
+        if os.path.exists(lib):
+            os.remove(lib)          # compile even if make would call the old library current
         compile_build(f"{output_dir}/build")
     return lib
 

@@ -44,14 +44,18 @@ def default_schedule(meta: MetaData, mean_bag_len: float = 1.0,
                      block_threads: int = 256) -> Tuple[ScheduleBase, NamedTuple]:
     """Untuned starting point for one feature from its row size and mean bag length: enough
     column lanes that a lane owns one or two 16-byte vectors, lookup lanes only for long bags,
-    and four to eight independent row loads in flight per lane."""
+    and two to four independent row loads in flight per lane -- fewer for fp16 and int8 rows,
+    whose 8 or 16 fp32 accumulators per 16-byte vector would otherwise push the fused kernel past
+    the registers that four or five workgroups per CU leave it (measured on C4 and C5: 2 % and
+    17 % faster than with four loads in flight everywhere)."""
     v = meta.row_vectors
     x = min(64, next_pow2(v))
     if v > 1 and x * meta.vec_bytes >= 256 and mean_bag_len < 8:
         x //= 2                      # short bags of wide rows: two vectors per lane
     vpl = -(-v // x)
+    acc_floats = vpl * meta.elems_per_vector          # accumulators of one bag per lane
     if mean_bag_len <= 1.5:
-        bags = 4 if vpl == 1 else 2
+        bags = 4 if 4 * acc_floats <= 16 else (2 if 2 * acc_floats <= 16 else 1)
         team = x
         if team == 1:
             return ThreadPerBagSchedule(meta, block_threads), ThreadPerBagParams(1, bags, vpl)
@@ -59,7 +63,7 @@ def default_schedule(meta: MetaData, mean_bag_len: float = 1.0,
             return WavefrontPerBagSchedule(meta, block_threads), WavefrontPerBagParams(64, 1, vpl)
         return (SubWavefrontPerBagSchedule(meta, block_threads),
                 SubWavefrontPerBagParams(x, 1, 1, bags, vpl))
-    items = 4 if vpl <= 2 else 2
+    items = 4 if acc_floats <= 8 else 2
     if mean_bag_len < 24:
         y = 1
     elif mean_bag_len < 96:
