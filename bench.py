@@ -50,6 +50,8 @@ def parse_args():
     p.add_argument("--copy-calibration", type=int, default=0,
                    help="also launch one plain device-to-device copy of this many bytes (for "
                         "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    p.add_argument("--no-gather-floor", action="store_true",
+                   help="skip the gather probe (bare fetch of the same rows, no sums, no output)")
     p.add_argument("--cpu-features", type=int, default=0,
                    help="bound the CPU leg to this many features (0 = choose from the size)")
     return p.parse_args()
@@ -125,7 +127,8 @@ def cpu_leg(wl, tables, indices, offsets, gpu_out, max_features: int):
 
 
 def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: int,
-               grid_blocks: int, cpu_features: int, xcd_segments: int = 0) -> dict:
+               grid_blocks: int, cpu_features: int, xcd_segments: int = 0,
+               gather_floor: bool = True) -> dict:
     import torch
     from recflex_amd import prebuilt
     from recflex_amd.rec_modules import FeatEmbed
@@ -195,6 +198,16 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
         "grid_blocks": grid_blocks or layer.max_concurrent_blocks,
         "setup_s": round(setup_s, 2),
     }
+    if gather_floor:
+        # the memory system's floor for this batch: the same rows fetched and dropped
+        from recflex_amd.gather_probe import GatherProbe
+        from recflex_amd.workloads import row_stride
+        probe = GatherProbe(dev, tables, d_idx, [row_stride(f.dim, f.data_type) for f in wl.features])
+        floor = probe.best_time_us(steps=min(steps, 10))
+        res["gather_floor_us"] = floor["us"]
+        res["gather_floor_setting"] = {k: v for k, v in floor.items() if k != "us"}
+        res["kernel_over_gather_floor"] = kernel_us_avg / floor["us"]
+        del probe
     if with_cpu:
         res["cpu_baseline"], res["check"] = cpu_leg(wl, tables, indices, offsets,
                                                     out, cpu_features)
@@ -224,14 +237,15 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
+    floor = not args.no_gather_floor
     head = run_config(args.workload, args.steps, args.warmup, not args.no_cpu, args.tile_bytes,
-                      args.grid_blocks, args.cpu_features, args.xcd_segments)
+                      args.grid_blocks, args.cpu_features, args.xcd_segments, floor)
     others = {}
     for name in [n for n in args.also.split(",") if n and n != args.workload]:
         try:
             others[name] = run_config(name, args.steps, args.warmup, not args.no_cpu,
                                       args.tile_bytes, args.grid_blocks, args.cpu_features,
-                                      args.xcd_segments)
+                                      args.xcd_segments, floor)
         except Exception as exc:  # a configuration that does not fit must not hide the headline
             others[name] = {"error": f"{type(exc).__name__}: {exc}"}
 
@@ -262,6 +276,10 @@ def main():
                      "traffic": MEASURED_TRAFFIC_BYTES.get(head["model"]), "kernel": "FusedKnl",
                      "algorithmic_bytes_per_launch": head["algorithmic_bytes"]},
     }
+    if "gather_floor_us" in head:
+        # time of the bare fetch of the same rows (gather probe): what the memory system allows
+        line["roofline"]["gather_floor_us"] = head["gather_floor_us"]
+        line["roofline"]["kernel_over_gather_floor"] = head["kernel_over_gather_floor"]
     if "cpu_baseline" in head:
         line["cpu_baseline"] = head["cpu_baseline"]
         line["check"] = head["check"]

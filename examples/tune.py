@@ -75,6 +75,9 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--xcd_segments_candidates", type=str,
                         help="comma-separated tile-walk settings swept in the global stage "
                              "(-1 = flat, n > 0 = n segments per XCD)")
+    parser.add_argument("--no_register_census", action="store_true", default=False,
+                        help="in-model local stage: admit every candidate to every occupancy's "
+                             "tournament, also those that spill registers there")
     parser.add_argument("--interference", type=str, default="model", choices=["model", "replicate"],
                         help="local stage: candidates timed inside the whole model, or per feature "
                              "against copies of themselves (the reference's scheme)")
@@ -137,7 +140,7 @@ def create_tune_config(args: argparse.Namespace) -> TuneConfig:
         occupancies = [int(v) for v in args.occupancies.split(",")]
     else:
         occupancies = list(range(1, max_threads_per_sm // args.block_threads + 1))
-    kwargs = {}
+    kwargs = {"register_census": not args.no_register_census}
     if args.tile_bytes:
         kwargs["tile_bytes"] = args.tile_bytes
     if args.xcd_segments_candidates:

@@ -81,6 +81,12 @@ class TuneConfig(NamedTuple):
     top_k: int = 8
     # passes of the whole-kernel climb that follows the tile-time tournament (0 = none)
     climb_passes: int = 1
+    # in-model local stage: compile every distinct candidate body alone for each occupancy and
+    # keep out of that occupancy's tournament the ones that spill or come within
+    # ``census_margin`` vector registers of the occupancy's budget (they cannot win, and their
+    # scratch memory and registers slow every other candidate of the same kernel down)
+    register_census: bool = True
+    census_margin: int = 8
     # global stage: traffic-per-tile values of the run-time binding to try for every occupancy
     # (a launch parameter, no rebuild); empty = only tile_bytes
     tile_bytes_candidates: List[int] = []
@@ -305,14 +311,95 @@ class Tuner:
         output_dir = f"{self.basic.codegen_dir}/tournament/o{occupancy}"
         return output_dir, f"{output_dir}/build"
 
+    # ---- register census ----------------------------------------------------------------------
+
+    @staticmethod
+    def vgpr_budget(occupancy: int) -> int:
+        """Vector registers per lane that ``occupancy`` 256-thread workgroups per CU (one
+        wavefront per SIMD each) leave a kernel on gfx950: 512 per SIMD in blocks of 8."""
+        return min(512, 512 // max(1, occupancy) // 8 * 8)
+
+    def _census_one(self, sched_param: Tuple[ScheduleBase, NamedTuple], occupancy: int,
+                    tune_config: TuneConfig) -> Tuple[int, int]:
+        """(vector registers, scratch bytes) of the fused kernel holding this one schedule."""
+        import re
+        import subprocess
+        import tempfile
+        from recflex_amd.code_emitter.build_basic import BasicBuilder
+        basic = BasicBuilder()
+        with tempfile.TemporaryDirectory(prefix="rfx_census_") as tmp:
+            src = f"{tmp}/process.hip"
+            CodeEmitter([sched_param]).emit(src, occupancy=occupancy, inline=tune_config.inline,
+                                            tile_bytes=tune_config.tile_bytes)
+            flags = [f for f in basic.hip_flags if f not in ("-shared", "-fPIC")]
+            cmd = [basic.hipcc, *flags, "-O3", f"-I{basic.include}", f"-I{basic.abi_include}",
+                   *(f"-I{inc}" for inc in self.basic.includes),
+                   "--cuda-device-only", "-S", "-o", f"{tmp}/process.s", src]
+            subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+            with open(f"{tmp}/process.s") as f:
+                text = f.read()
+        vgprs = max(int(v) for v in re.findall(r"; NumVgprs: (\d+)", text))
+        scratch = max(int(v) for v in re.findall(r"; ScratchSize: (\d+)", text))
+        return vgprs, scratch
+
+    def register_census(self, occupancy: int, tune_config: TuneConfig) -> Dict[str, Tuple[int, int]]:
+        """Registers and scratch of every distinct candidate body at this occupancy, keyed by the
+        body text; compiled once (``.cache/census_o{occ}.json``), ``num_processes`` at a time."""
+        from concurrent.futures import ThreadPoolExecutor
+        cache_path = f"{self.basic.codegen_dir}/.cache/census_o{occupancy}.json"
+        census: Dict[str, Tuple[int, int]] = {}
+        if os.path.exists(cache_path) and not tune_config.recompile:
+            with open(cache_path) as f:
+                census = {k: tuple(v) for k, v in json.load(f).items()}
+        todo: Dict[str, Tuple[ScheduleBase, NamedTuple]] = {}
+        for cands in self.feat_sched_param_candidates:
+            for sched, params in cands:
+                key = hashlib.sha256(sched.EmitScheduleBody(params).encode()).hexdigest()[:24]
+                if key not in census:
+                    todo.setdefault(key, (sched, params))
+        if todo:
+            print(f"register census, occupancy {occupancy}: {len(todo)} schedule bodies", flush=True)
+            with ThreadPoolExecutor(max_workers=max(1, tune_config.num_processes)) as pool:
+                done = pool.map(lambda sp: self._census_one(sp, occupancy, tune_config), todo.values())
+                for key, res in zip(todo.keys(), done):
+                    census[key] = res
+            os.makedirs(os.path.dirname(cache_path), exist_ok=True)
+            with open(cache_path, "w") as f:
+                json.dump(census, f)
+        return census
+
+    def tournament_candidates(self, occupancy: int, tune_config: TuneConfig) -> List[List[int]]:
+        """Per feature, the indices (into its candidate list) admitted to this occupancy's
+        tournament: bodies that do not spill and stay ``census_margin`` registers under the
+        occupancy's budget; the lightest body of the feature if none does."""
+        if not tune_config.register_census:
+            return [list(range(len(c))) for c in self.feat_sched_param_candidates]
+        census = self.register_census(occupancy, tune_config)
+        limit = self.vgpr_budget(occupancy) - tune_config.census_margin
+        admitted = []
+        for cands in self.feat_sched_param_candidates:
+            stats = [census[hashlib.sha256(s.EmitScheduleBody(p).encode()).hexdigest()[:24]]
+                     for s, p in cands]
+            keep = [k for k, (vgprs, scratch) in enumerate(stats) if scratch == 0 and vgprs <= limit]
+            if not keep:
+                keep = [min(range(len(stats)), key=lambda k: (stats[k][1], stats[k][0]))]
+            admitted.append(keep)
+        return admitted
+
     def compile_tournament(self, tune_config: TuneConfig) -> None:
-        """One timing build of the whole model per occupancy, holding all candidates."""
+        """One timing build of the whole model per occupancy, holding the admitted candidates;
+        ``admitted.json`` beside it maps its candidate numbers back to the full lists."""
         jobs = []
         for occupancy in tune_config.occupancies:
             output_dir, build_dir = self.get_tournament_dir(occupancy)
             if not os.path.exists(f"{build_dir}/librecom.so") or tune_config.recompile:
                 os.makedirs(build_dir, exist_ok=True)
-                emitter = CodeEmitter(None, feat_candidates=self.feat_sched_param_candidates)
+                admitted = self.tournament_candidates(occupancy, tune_config)
+                with open(f"{output_dir}/admitted.json", "w") as f:
+                    json.dump(admitted, f)
+                cands = [[self.feat_sched_param_candidates[feat][k] for k in keep]
+                         for feat, keep in enumerate(admitted)]
+                emitter = CodeEmitter(None, feat_candidates=cands)
                 emitter.emit(f"{output_dir}/process.hip", occupancy=occupancy, timing=True,
                              inline=tune_config.inline, tune=True, tile_bytes=tune_config.tile_bytes)
                 emitter.emit_cmake_list(f"{output_dir}/CMakeLists.txt", code_fname="process.hip",
@@ -321,6 +408,14 @@ class Tuner:
                                         debug=tune_config.debug)
                 jobs.append((output_dir, build_dir))
         self._schedule_builds(jobs, tune_config)
+
+    def admitted_candidates(self, occupancy: int) -> List[List[int]]:
+        output_dir, _ = self.get_tournament_dir(occupancy)
+        path = f"{output_dir}/admitted.json"
+        if not os.path.exists(path):
+            return [list(range(len(c))) for c in self.feat_sched_param_candidates]
+        with open(path) as f:
+            return json.load(f)
 
     def default_choices(self) -> List[List[int]]:
         """Index, in every feature's candidate list, of the schedule ``default_schedule`` would
@@ -353,10 +448,12 @@ class Tuner:
             output_dir, build_dir = self.get_tournament_dir(occupancy)
             result_log = f"{output_dir}/result.json"
             if not os.path.exists(result_log) or tune_config.remeasure:
+                admitted = self.admitted_candidates(occupancy)
+                starts = [[self._nearest_admitted(feat, pick, admitted[feat])
+                           for feat, pick in enumerate(choice)] for choice in self.default_choices()]
                 args = (occupancy, f"{build_dir}/librecom.so", self.table_shapes, self.data_types,
                         self.data_npzs, result_log, tune_config.rounds, tune_config.refine_passes,
-                        tune_config.top_k, 0.2, 3, 0, tune_config.climb_passes,
-                        self.default_choices())
+                        tune_config.top_k, 0.2, 3, 0, tune_config.climb_passes, starts)
                 self._run_measure(manager, tune_config, measure_tournament, args)
         if manager:
             manager.join()
@@ -365,9 +462,29 @@ class Tuner:
             output_dir, _ = self.get_tournament_dir(occupancy)
             with open(f"{output_dir}/result.json") as f:        # absent if the worker failed
                 times = json.load(f)["times"]
+            admitted = self.admitted_candidates(occupancy)
             for feat_id in range(self.num_feats):
-                results[feat_id][occupancy] = times[feat_id]
+                # candidates kept out of this occupancy's tournament never win it
+                full = [float("inf")] * len(self.feat_sched_param_candidates[feat_id])
+                for k, t in zip(admitted[feat_id], times[feat_id]):
+                    full[k] = t
+                results[feat_id][occupancy] = full
         return results
+
+    def _nearest_admitted(self, feat_id: int, pick: int, admitted: List[int]) -> int:
+        """Position, in the admitted list, of candidate ``pick`` of the feature -- or of the
+        admitted candidate of the same template closest to it in parameters."""
+        if pick in admitted:
+            return admitted.index(pick)
+        cands = self.feat_sched_param_candidates[feat_id]
+        sched, params = cands[pick]
+
+        def distance(k: int) -> Tuple[int, int]:
+            s, p = cands[k]
+            if type(s) is not type(sched):
+                return (1, 0)
+            return (0, sum(abs(a - b) for a, b in zip(p, params)))
+        return min(range(len(admitted)), key=lambda j: distance(admitted[j]))
 
     def tune(self, tune_config: TuneConfig) -> Dict[int, Dict[int, List[float]]]:
         if tune_config.interference == "model":

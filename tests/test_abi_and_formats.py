@@ -178,3 +178,17 @@ def test_rocprof_stats_reader(tmp_path):
     assert parse_first_knl_total_time(str(tmp_path)) == 1500000
     with pytest.raises(FileNotFoundError):
         parse_knl_total_time("FusedKnl", str(tmp_path / "nothing_here"))
+
+
+def test_gather_probe_chunks_cover_every_lookup_once():
+    from recflex_amd.gather_probe import make_chunks, CHUNK_LOOKUPS
+    lookups = [2500, 0, 10, 1024]
+    vectors = [2, 9, 64, 1]
+    chunks = make_chunks(lookups, vectors)
+    assert chunks.dtype == np.int32 and chunks.shape[1] == 4
+    for f, n in enumerate(lookups):
+        mine = chunks[chunks[:, 0] == f]
+        assert mine[:, 2].sum() == n and (mine[:, 2] <= CHUNK_LOOKUPS).all() and (mine[:, 2] > 0).all()
+        assert list(mine[:, 1]) == list(range(0, n, CHUNK_LOOKUPS))
+        assert all(1 << int(l) >= min(vectors[f], 64) for l in mine[:, 3])
+    assert make_chunks([0, 0], [1, 1]).shape == (0, 4)

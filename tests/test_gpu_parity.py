@@ -82,3 +82,26 @@ def test_onehot_is_bit_exact():
     """Bags of exactly one lookup are a row copy: identical bits (C2 shape, shrunk)."""
     wl, got, want = _run_model("c2s")
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_gather_probe_runs():
+    """The measurement aid of bench.py: fetches the rows of a batch and nothing else.  It must
+    run to completion on ragged inputs (empty features, rows of 1 to 64 vectors) and take time."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.gather_probe import GatherProbe
+    from recflex_amd.workloads import gen_inputs, gen_tables, row_stride
+
+    wl = prebuilt.model_spec("edge").workload
+    dev = torch.device("cuda", 0)
+    print(f"[case] gather probe on edge: F={wl.num_features} B={wl.batch}", flush=True)
+    tables = gen_tables(wl, dev)
+    indices, _ = gen_inputs(wl)
+    d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+    probe = GatherProbe(dev, tables, d_idx, [row_stride(f.dim, f.data_type) for f in wl.features])
+    strides = [row_stride(f.dim, f.data_type) for f in wl.features]
+    assert probe.n_chunks == sum(-(-len(i) // 1024) for i, s in zip(indices, strides) if s >= 16)
+    for kwargs in ({"in_flight": 2}, {"in_flight": 8, "segments": 16}, {"workgroups_per_cu": 3, "segments": 2}):
+        assert probe.time_us(steps=3, warmup=1, **kwargs) > 0
+    best = probe.best_time_us(steps=2)
+    assert best["us"] > 0 and best["in_flight"] in (2, 4, 8)
