@@ -75,6 +75,11 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--xcd_segments_candidates", type=str,
                         help="comma-separated tile-walk settings swept in the global stage "
                              "(-1 = flat, n > 0 = n segments per XCD)")
+    parser.add_argument("--build_climb_trials", type=int, default=0,
+                        help="global stage: that many single-feature variants of the winning mix are "
+                             "built as production kernels and timed; the faster ones are adopted")
+    parser.add_argument("--build_climb_top_k", type=int, default=3,
+                        help="build climb: tournament candidates tried per feature")
     parser.add_argument("--no_register_census", action="store_true", default=False,
                         help="in-model local stage: admit every candidate to every occupancy's "
                              "tournament, also those that spill registers there")
@@ -140,7 +145,9 @@ def create_tune_config(args: argparse.Namespace) -> TuneConfig:
         occupancies = [int(v) for v in args.occupancies.split(",")]
     else:
         occupancies = list(range(1, max_threads_per_sm // args.block_threads + 1))
-    kwargs = {"register_census": not args.no_register_census}
+    kwargs = {"register_census": not args.no_register_census,
+              "build_climb_trials": args.build_climb_trials,
+              "build_climb_top_k": args.build_climb_top_k}
     if args.tile_bytes:
         kwargs["tile_bytes"] = args.tile_bytes
     if args.xcd_segments_candidates:

@@ -2,7 +2,7 @@
 
 Measurement aid for ``bench.py``: the same tables and index streams as the fused kernel, 16-byte
 loads, no sums and no output, swept over the loads in flight per lane, the resident workgroups
-per CU, the chunk size and the XCD-segmented walk; the fastest setting is reported.  Its time is
+per CU, the bytes per chunk and the XCD-segmented walk; the fastest setting is reported.  Its time is
 what the memory system (HBM, Infinity Cache, L2, L1 miss handling) needs for the rows of this
 batch alone.
 """
@@ -17,10 +17,10 @@ import numpy as np
 from recflex_amd.code_emitter.build_basic import BasicBuilder
 
 CHUNK_LOOKUPS = 1024
-SWEEP_IN_FLIGHT = (2, 4, 8)
+SWEEP_IN_FLIGHT = (4, 8)
 SWEEP_WORKGROUPS_PER_CU = (4, 8)
-SWEEP_SEGMENTS = (0, 16)
-SWEEP_CHUNK_LOOKUPS = (256, 1024)
+SWEEP_SEGMENTS = (0, 16, 32)
+SWEEP_CHUNK_BYTES = (16384, 65536)
 
 
 def lib_path() -> str:
@@ -40,13 +40,15 @@ def build(force: bool = False) -> str:
 
 
 def make_chunks(num_lookups: Sequence[int], row_vectors: Sequence[int],
-                chunk_lookups: int = CHUNK_LOOKUPS) -> np.ndarray:
+                chunk_lookups: int = CHUNK_LOOKUPS, chunk_bytes: int = 0) -> np.ndarray:
     """int32 [n, 4] records (feat, begin, count, log2 of the lanes per row), ordered by feature
-    like the fused kernel's tile space."""
+    like the fused kernel's tile space.  ``chunk_bytes`` > 0 sizes the chunks of every feature to
+    about that many row bytes (32..4096 lookups) instead of ``chunk_lookups`` lookups."""
     out: List[tuple] = []
     for f, (n, v) in enumerate(zip(num_lookups, row_vectors)):
         log2x = min(6, max(0, int(np.ceil(np.log2(max(1, v))))))
-        out.extend((f, b, min(chunk_lookups, n - b), log2x) for b in range(0, n, chunk_lookups))
+        per = max(32, min(4096, chunk_bytes // (16 * max(1, v)))) if chunk_bytes > 0 else chunk_lookups
+        out.extend((f, b, min(per, n - b), log2x) for b in range(0, n, per))
     return np.asarray(out, dtype=np.int32).reshape(-1, 4)
 
 
@@ -76,9 +78,9 @@ class GatherProbe:
         self.cus = torch.cuda.get_device_properties(device).multi_processor_count
         self.set_chunks(CHUNK_LOOKUPS)
 
-    def set_chunks(self, chunk_lookups: int) -> None:
+    def set_chunks(self, chunk_lookups: int = CHUNK_LOOKUPS, chunk_bytes: int = 0) -> None:
         import torch
-        chunks = make_chunks(self.num_lookups, self.row_vectors, chunk_lookups)
+        chunks = make_chunks(self.num_lookups, self.row_vectors, chunk_lookups, chunk_bytes)
         self.n_chunks = len(chunks)
         self.d_chunks = torch.from_numpy(chunks).to(self.device) if len(chunks) else \
             torch.zeros((1, 4), dtype=torch.int32, device=self.device)
@@ -111,15 +113,15 @@ class GatherProbe:
 
     def best_time_us(self, steps: int = 10) -> dict:
         """Sweeps the settings; returns the fastest as {"us", "in_flight", "workgroups_per_cu",
-        "segments", "chunk_lookups"}."""
+        "segments", "chunk_bytes"}."""
         best = None
-        for chunk in SWEEP_CHUNK_LOOKUPS:
-            self.set_chunks(chunk)
+        for chunk in SWEEP_CHUNK_BYTES:
+            self.set_chunks(chunk_bytes=chunk)
             for u in SWEEP_IN_FLIGHT:
                 for occ in SWEEP_WORKGROUPS_PER_CU:
                     for seg in SWEEP_SEGMENTS:
                         t = self.time_us(steps=steps, in_flight=u, workgroups_per_cu=occ, segments=seg)
                         if best is None or t < best["us"]:
                             best = {"us": t, "in_flight": u, "workgroups_per_cu": occ,
-                                    "segments": seg, "chunk_lookups": chunk}
+                                    "segments": seg, "chunk_bytes": chunk}
         return best

@@ -369,6 +369,41 @@ def measure_kernel_events(librecom_path: str, table_shapes: Sequence[Tuple[int, 
         return None
 
 
+class KernelTimer:
+    """Times the FusedKnl of several libraries of one model over the same tables and batches,
+    which stay on the device between calls (the production-build climb times hundreds of
+    libraries; building the tables anew for each would cost more than the measurements)."""
+
+    def __init__(self, table_shapes: Sequence[Tuple[int, int]], data_types: Sequence[str],
+                 data_npzs: Sequence[str], gpu_id: int = None):
+        _pin_gpu(gpu_id)
+        import torch
+        self.dev = torch.device("cuda", torch.cuda.current_device())
+        self.tables = [make_table(s, t, self.dev, ones=False) for s, t in zip(table_shapes, data_types)]
+        per_feat = [load_batches(p) for p in data_npzs]
+        self.batches = []
+        for k in range(len(per_feat[0])):
+            self.batches.append(([torch.from_numpy(b[k][0]).to(self.dev) for b in per_feat],
+                                 [torch.from_numpy(b[k][1]).to(self.dev) for b in per_feat]))
+        self.outs = None
+
+    def time_ns(self, librecom_path: str, tile_bytes: int = 0, xcd_segments: int = 0,
+                repeats: int = 7, warmup: int = 4) -> float:
+        """Sum over the batches of the median time per launch, in ns."""
+        from recflex_amd.rec_modules import FeatEmbed
+        layer = FeatEmbed(self.dev, embed_tables=self.tables, librecom=librecom_path)
+        if self.outs is None:
+            self.outs = [layer.forward_indices(d_idx, d_off).clone() for d_idx, d_off in self.batches]
+        total = 0.0
+        for (d_idx, d_off), out in zip(self.batches, self.outs):
+            run = lambda: layer.forward_indices(d_idx, d_off, out=out, tile_bytes=tile_bytes,
+                                                xcd_segments=xcd_segments)
+            for _ in range(warmup):
+                run()
+            total += _timed_launches(run, repeats)
+        return total
+
+
 MAX_TILE_FACTOR = 8      # rfx::kMaxTileFactor
 
 

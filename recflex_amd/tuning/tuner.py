@@ -39,7 +39,7 @@ from recflex_amd.parser import (parse_raw_data_batches, parse_table_shapes, pars
 
 from .measure import (measure_single_feat, rocprof_profile, measure_task_blocks,
                       measure_naive_candidate, measure_kernel_events, measure_tournament,
-                      save_batches)
+                      save_batches, KernelTimer)
 
 
 class BasicConfig(NamedTuple):
@@ -87,6 +87,14 @@ class TuneConfig(NamedTuple):
     # scratch memory and registers slow every other candidate of the same kernel down)
     register_census: bool = True
     census_margin: int = 8
+    # global stage, after the contenders are timed: hill climb on production builds.  The
+    # winning mix is varied one feature at a time (heaviest first, that feature's
+    # ``build_climb_top_k`` best tournament candidates), ``num_processes`` variants are compiled
+    # side by side and timed as whole kernels, and the variants that are faster are adopted.
+    # 0 trials = off; the budget bounds the compile time spent
+    build_climb_trials: int = 0
+    build_climb_top_k: int = 3
+    build_climb_min_gain: float = 0.01
     # global stage: traffic-per-tile values of the run-time binding to try for every occupancy
     # (a launch parameter, no rebuild); empty = only tile_bytes
     tile_bytes_candidates: List[int] = []
@@ -534,7 +542,15 @@ class Tuner:
         shutil.copytree(output_dir, optimal)
         tile_bytes = getattr(self, "opt_tile_bytes", tune_config.tile_bytes)
         xcd_segments = getattr(self, "opt_xcd_segments", 0)
-        if tile_bytes != tune_config.tile_bytes or xcd_segments:
+        climbed = False
+        if tune_config.build_climb_trials > 0:
+            mix, t = self.build_climb(opt_sched_params, opt_occupancy, measured_times, tune_config,
+                                      tile_bytes=tile_bytes, xcd_segments=xcd_segments)
+            climbed = any(a[0].EmitScheduleBody(a[1]) != b[0].EmitScheduleBody(b[1])
+                          for a, b in zip(mix, opt_sched_params))
+            opt_sched_params = mix
+            print(f"occupancy: {opt_occupancy} (after the build climb), t(ns): {t}", flush=True)
+        if climbed or tile_bytes != tune_config.tile_bytes or xcd_segments:
             # make the winning launch parameters the defaults of the optimal library
             self.emit_codes(output_dir=optimal, feat_schedules=opt_sched_params, occupancy=opt_occupancy,
                             inline=tune_config.inline, debug=tune_config.debug, tile_bytes=tile_bytes,
@@ -657,6 +673,130 @@ class Tuner:
         self.opt_xcd_segments = best_opts[opt_idx][1]
         self.opt_output_dir, opt_occupancy, opt_sched_params = contenders[opt_idx]
         return opt_occupancy, opt_sched_params
+
+    def build_climb(self, start: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
+                    measured_times: Dict[int, Dict[int, List[float]]], tune_config: TuneConfig,
+                    tile_bytes: int = 0, xcd_segments: int = 0
+                    ) -> Tuple[List[Tuple[ScheduleBase, NamedTuple]], float]:
+        """Hill climb on production builds (see ``TuneConfig.build_climb_trials``).  Tile times and
+        even whole-kernel times taken inside the tournament build do not carry over exactly to a
+        production build (other register allocation, other code size), so the last word goes to
+        kernels built exactly as they ship.  Returns the improved mix and its time in ns."""
+        climb_dir = f"{self.basic.codegen_dir}/climb/o{occupancy}"
+        timer = KernelTimer(self.table_shapes, self.data_types, self.data_npzs,
+                            gpu_id=tune_config.gpu_ids[0])
+        cfg = tune_config._replace(tile_bytes=tile_bytes or tune_config.tile_bytes)
+
+        def build_all(mixes: List[Tuple[str, list]]) -> None:
+            jobs = []
+            for name, mix in mixes:
+                out = f"{climb_dir}/{name}"
+                if not os.path.exists(f"{out}/build/librecom.so"):
+                    os.makedirs(f"{out}/build", exist_ok=True)
+                    self.emit_codes(output_dir=out, feat_schedules=mix, occupancy=occupancy,
+                                    inline=cfg.inline, debug=cfg.debug, tile_bytes=cfg.tile_bytes,
+                                    host=False, xcd_segments=max(xcd_segments, 0))
+                    jobs.append((out, f"{out}/build"))
+            self._schedule_builds(jobs, cfg)
+
+        def time_of(name: str, repeats: int = 7) -> float:
+            return timer.time_ns(f"{climb_dir}/{name}/build/librecom.so", repeats=repeats)
+
+        best = list(start)
+        build_all([("base0", best)])
+        best_ns = time_of("base0", repeats=11)
+        print(f"[build climb {occupancy}] start {best_ns:.0f} ns", flush=True)
+
+        # Moves, heaviest first.  Group moves: all features that run the same body now (and have
+        # the same candidate list) switch together to one of the candidates their summed
+        # tournament scores rank best -- a change too small to measure on one light feature shows
+        # when twenty features make it.  Then single-feature moves.
+        lookups = [sum(len(i) for i, _ in self.batches[f]) for f in range(self.num_feats)]
+        weight = np.asarray([lookups[f] * self.metas[f].row_bytes + self.metas[f].embed_dim * 4 *
+                             sum(len(o) - 1 for _, o in self.batches[f])
+                             for f in range(self.num_feats)], dtype=np.float64)
+        top_k = tune_config.build_climb_top_k
+
+        def scores_of(feat: int) -> np.ndarray:
+            return np.asarray(measured_times[feat][occupancy], dtype=np.float64)
+
+        groups: Dict[Tuple[str, int], List[int]] = {}
+        for feat in range(self.num_feats):
+            key = (best[feat][0].EmitScheduleBody(best[feat][1]), len(self.feat_sched_param_candidates[feat]))
+            groups.setdefault(key, []).append(feat)
+        moves: List[Tuple[List[int], int]] = []
+        for feats in sorted(groups.values(), key=lambda g: -weight[g].sum()):
+            if len(feats) < 2:
+                continue
+            ref = self.feat_sched_param_candidates[feats[0]]
+            same = all(all(a[0].EmitScheduleBody(a[1]) == b[0].EmitScheduleBody(b[1])
+                           for a, b in zip(ref, self.feat_sched_param_candidates[f])) for f in feats[1:])
+            if not same:
+                continue
+            total = np.zeros(len(ref))
+            for f in feats:
+                sc = scores_of(f)
+                finite = sc[np.isfinite(sc)]
+                total += np.where(np.isfinite(sc), sc / (finite.min() if finite.size else 1.0), np.inf)
+            ranked = [int(k) for k in np.argsort(total) if np.isfinite(total[k])]
+            moves.extend((list(feats), k) for k in ranked[:top_k])
+        for feat in np.argsort(-weight):
+            sc = scores_of(int(feat))
+            ranked = [int(k) for k in np.argsort(sc) if np.isfinite(sc[k])]
+            moves.extend(([int(feat)], k) for k in ranked[:top_k])
+        moves = moves[:tune_config.build_climb_trials]
+
+        def body(cand) -> str:
+            return cand[0].EmitScheduleBody(cand[1])
+
+        width = max(1, tune_config.num_processes)
+        generation = 0
+        for lo in range(0, len(moves), width):
+            batch = []
+            for j, (feats, k) in enumerate(moves[lo:lo + width]):
+                mix = list(best)
+                for f in feats:
+                    mix[f] = self.feat_sched_param_candidates[f][k]
+                if all(body(mix[f]) == body(best[f]) for f in feats):
+                    continue
+                batch.append((f"g{generation}_m{lo + j}", feats, k, mix))
+            if not batch:
+                continue
+            build_all([(name, mix) for name, _, _, mix in batch])
+            gains = []
+            for name, feats, k, _ in batch:
+                t = time_of(name)
+                if t < best_ns * (1.0 - tune_config.build_climb_min_gain):
+                    gains.append((t, feats, k, name))
+            if not gains:
+                continue
+            gains.sort(key=lambda g: g[0])
+            # several moves may have helped: adopt those that touch different features together
+            # if that is faster still
+            merged = list(best)
+            taken: set = set()
+            adopted = 0
+            for _, feats, k, _ in gains:
+                if taken.isdisjoint(feats):
+                    for f in feats:
+                        merged[f] = self.feat_sched_param_candidates[f][k]
+                    taken.update(feats)
+                    adopted += 1
+            generation += 1
+            t_single = time_of(gains[0][3], repeats=11)
+            t_merged = t_single
+            if adopted > 1:
+                build_all([(f"base{generation}", merged)])
+                t_merged = time_of(f"base{generation}", repeats=11)
+            if adopted > 1 and t_merged <= t_single and t_merged < best_ns:
+                best, best_ns = merged, t_merged
+            elif t_single < best_ns:
+                best = list(best)
+                for f in gains[0][1]:
+                    best[f] = self.feat_sched_param_candidates[f][gains[0][2]]
+                best_ns = t_single
+            print(f"[build climb {occupancy}] after {lo + len(batch)} moves: {best_ns:.0f} ns", flush=True)
+        return best, best_ns
 
     # ------------------------------------------------------------------ validation / ablations
 

@@ -192,3 +192,9 @@ def test_gather_probe_chunks_cover_every_lookup_once():
         assert list(mine[:, 1]) == list(range(0, n, CHUNK_LOOKUPS))
         assert all(1 << int(l) >= min(vectors[f], 64) for l in mine[:, 3])
     assert make_chunks([0, 0], [1, 1]).shape == (0, 4)
+    by_bytes = make_chunks(lookups, vectors, chunk_bytes=16384)
+    for f, n in enumerate(lookups):
+        mine = by_bytes[by_bytes[:, 0] == f]
+        assert mine[:, 2].sum() == n
+        if n:
+            assert mine[0, 2] == min(n, max(32, min(4096, 16384 // (16 * vectors[f]))))

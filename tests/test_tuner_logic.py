@@ -186,3 +186,94 @@ def test_task_manager_returns_resources_and_survives_failures(tmp_path):
     assert len(lines) == 5 and set(lines) <= {"gpu0", "gpu1"}
     assert tm.resource_queue.qsize() == 2          # both resources are back
     assert sorted(tm.exit_codes) == [0, 0, 0, 0, 0, 1]
+
+
+def test_register_census_filters_the_tournament(tmp_path, monkeypatch):
+    """Candidates that spill, or come within the margin of the occupancy's register budget, stay
+    out of that occupancy's tournament; results are mapped back to the full candidate lists."""
+    t = _tiny_tuner(tmp_path)
+    assert [Tuner.vgpr_budget(o) for o in (1, 2, 3, 4, 5, 6, 8)] == [512, 256, 168, 128, 96, 80, 64]
+    cfg = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=2, in_process=True)
+
+    def fake_census(sched_param, occupancy, tune_config):      # no compiler in this test
+        params = sched_param[1]
+        heavy = sum(params) % 3 == 0
+        return (124 if heavy else 60 + sum(params) % 40, 64 if sum(params) % 5 == 0 else 0)
+
+    monkeypatch.setattr(t, "_census_one", fake_census)
+    admitted = t.tournament_candidates(4, cfg)
+    for feat, keep in enumerate(admitted):
+        cands = t.feat_sched_param_candidates[feat]
+        assert keep and keep == sorted(keep)
+        for k, cand in enumerate(cands):
+            vgprs, scratch = fake_census(cand, 4, cfg)
+            assert (k in keep) == (scratch == 0 and vgprs <= 128 - cfg.census_margin)
+    assert os.path.exists(f"{t.basic.codegen_dir}/.cache/census_o4.json")
+    # a second call reads the cache
+    monkeypatch.setattr(t, "_census_one", lambda *a: (_ for _ in ()).throw(AssertionError("recompiled")))
+    assert t.tournament_candidates(4, cfg) == admitted
+    # nothing fits: the lightest body is admitted anyway
+    assert all(len(k) == 1 for k in t.tournament_candidates(4, cfg._replace(census_margin=128)))
+
+    out, build_dir = t.get_tournament_dir(4)
+    os.makedirs(build_dir, exist_ok=True)
+    open(f"{build_dir}/librecom.so", "wb").close()
+    with open(f"{out}/admitted.json", "w") as fh:
+        json.dump(admitted, fh)
+    with open(f"{out}/result.json", "w") as fh:
+        json.dump({"times": [[float(j + 1) for j in range(len(k))] for k in admitted]}, fh)
+    res = t.tune(cfg)
+    for feat, keep in enumerate(admitted):
+        full = res[feat][4]
+        assert len(full) == len(t.feat_sched_param_candidates[feat])
+        assert [full[k] for k in keep] == [float(j + 1) for j in range(len(keep))]
+        assert all(np.isinf(full[k]) for k in range(len(full)) if k not in keep)
+        assert t._nearest_admitted(feat, keep[-1], keep) == len(keep) - 1
+        assert 0 <= t._nearest_admitted(feat, 0, keep) < len(keep)
+
+
+def test_build_climb_adopts_faster_production_builds(tmp_path, monkeypatch):
+    """The climb on production builds, with the compiler and the GPU replaced: a kernel's time is
+    the sum of a fixed cost per schedule body, so the optimum over the tried candidates is known."""
+    import recflex_amd.tuning.tuner as tuner_mod
+    t = _tiny_tuner(tmp_path)
+    occ = 4
+
+    def body_cost(cand) -> float:
+        text = cand[0].EmitScheduleBody(cand[1])
+        return 1000.0 + (sum(map(ord, text)) * 7919) % 500
+
+    def fake_builds(jobs, tune_config):
+        for out, build_dir in jobs:
+            os.makedirs(build_dir, exist_ok=True)
+            open(f"{build_dir}/librecom.so", "wb").close()
+
+    class FakeTimer:
+        def __init__(self, *a, **k):
+            pass
+
+        def time_ns(self, lib, repeats=7, **k):
+            entries = json.load(open(os.path.join(os.path.dirname(os.path.dirname(lib)), "schedule.json")))
+            from recflex_amd.schedules import schedule_from_config
+            return sum(body_cost(schedule_from_config(e, MetaData(e["embed_dim"], e.get("data_type", "float"))))
+                       for e in entries)
+
+    monkeypatch.setattr(t, "_schedule_builds", fake_builds)
+    monkeypatch.setattr(tuner_mod, "KernelTimer", FakeTimer)
+    cands = t.feat_sched_param_candidates
+    # tournament scores rank the candidates in list order; the start is each feature's last one
+    scores = {f: {occ: [float(k) for k in range(len(c))]} for f, c in enumerate(cands)}
+    start = [c[-1] for c in cands]
+    cfg = TuneConfig(occupancies=[occ], gpu_ids=[0], sm_count=4, num_processes=3, in_process=True,
+                     build_climb_trials=100, build_climb_top_k=4, build_climb_min_gain=0.001)
+    mix, t_ns = t.build_climb(start, occ, scores, cfg)
+    want = 0.0
+    for f, c in enumerate(cands):
+        tried = [c[-1]] + c[:4]
+        want += min(body_cost(x) for x in tried)
+        assert body_cost(mix[f]) == min(body_cost(x) for x in tried)
+    assert t_ns == pytest.approx(want)
+    assert t_ns <= sum(body_cost(x) for x in start)
+    # no trials: the start mix comes back with its own time
+    mix0, t0 = t.build_climb(start, occ, scores, cfg._replace(build_climb_trials=0))
+    assert mix0 == start and t0 == pytest.approx(sum(body_cost(x) for x in start))
