@@ -78,6 +78,9 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--build_climb_trials", type=int, default=0,
                         help="global stage: that many single-feature variants of the winning mix are "
                              "built as production kernels and timed; the faster ones are adopted")
+    parser.add_argument("--climb_passes", type=int, default=1,
+                        help="in-model local stage: passes of the whole-kernel climb inside the "
+                             "tournament build (0 = rank by tile time only)")
     parser.add_argument("--build_climb_top_k", type=int, default=3,
                         help="build climb: tournament candidates tried per feature")
     parser.add_argument("--no_register_census", action="store_true", default=False,
@@ -147,7 +150,8 @@ def create_tune_config(args: argparse.Namespace) -> TuneConfig:
         occupancies = list(range(1, max_threads_per_sm // args.block_threads + 1))
     kwargs = {"register_census": not args.no_register_census,
               "build_climb_trials": args.build_climb_trials,
-              "build_climb_top_k": args.build_climb_top_k}
+              "build_climb_top_k": args.build_climb_top_k,
+              "climb_passes": args.climb_passes}
     if args.tile_bytes:
         kwargs["tile_bytes"] = args.tile_bytes
     if args.xcd_segments_candidates:

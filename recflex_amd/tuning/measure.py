@@ -23,6 +23,7 @@ because ``TORCH_LIBRARY(recom)`` can be registered once (``measure.py:23-24``).
 """
 
 import json
+import time
 import os
 import shutil
 import subprocess
@@ -177,6 +178,13 @@ def measure_tournament(ident: int, librecom_path: str, table_shapes: Sequence[Tu
             device_batches.append(([torch.from_numpy(b[k][0]).to(dev) for b in per_feat],
                                    [torch.from_numpy(b[k][1]).to(dev) for b in per_feat]))
         rng = np.random.default_rng(seed)
+        last_beat = [time.monotonic()]
+
+        def beat(what: str) -> None:
+            """A progress line every 20 s or so: long phases of a large model are otherwise silent."""
+            if time.monotonic() - last_beat[0] > 20.0:
+                last_beat[0] = time.monotonic()
+                print(f"[tournament {ident}] {what}", flush=True)
 
         def launch(choice: np.ndarray) -> np.ndarray:
             d_choice = torch.from_numpy(choice.astype(np.int32)).to(dev)
@@ -196,6 +204,7 @@ def measure_tournament(ident: int, librecom_path: str, table_shapes: Sequence[Tu
             for j in range(steps):
                 choice = np.array([perms[f][j % counts[f]] for f in range(num_feats)])
                 t = launch(choice)
+                beat(f"exploration, step {j + 1} of {steps}")
                 for f in range(num_feats):
                     sums[f][choice[f]] += t[f]
                     hits[f][choice[f]] += 1
@@ -214,6 +223,7 @@ def measure_tournament(ident: int, librecom_path: str, table_shapes: Sequence[Tu
                 for f in np.nonzero(probing)[0]:
                     choice[f] = rng.choice(tops[f])
                 t = launch(choice)
+                beat("refinement")
                 for f in range(num_feats):
                     rsum[f][choice[f]] += t[f]
                     rhit[f][choice[f]] += 1
@@ -257,6 +267,7 @@ def measure_tournament(ident: int, librecom_path: str, table_shapes: Sequence[Tu
                         trial = best.copy()
                         trial[f] = c
                         t = kernel_ns(trial)
+                        beat(f"climb, best {best_ns:.0f} ns")
                         if t < best_ns * 0.995:
                             t = kernel_ns(trial, reps=5)     # confirm before keeping
                             if t < best_ns * 0.995:
