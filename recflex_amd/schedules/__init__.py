@@ -64,6 +64,14 @@ def default_schedule(meta: MetaData, mean_bag_len: float = 1.0,
         return (SubWavefrontPerBagSchedule(meta, block_threads),
                 SubWavefrontPerBagParams(x, 1, 1, bags, vpl))
     items = 4 if acc_floats <= 8 else 2
+    if mean_bag_len >= 96 and meta.payload_bytes >= 512 and vpl * meta.elems_per_vector < 16:
+        # long bags of wide rows: fewer column lanes, each with 16 accumulators (4 fp32 or 2 fp16
+        # vectors), so that four (two) times as many lookups are in flight per wavefront -- the
+        # move the production-build climb makes first on C3 (fp32, D=128) and C4 (fp16, D=256)
+        vpl = max(1, 16 // meta.elems_per_vector)
+        x = max(1, next_pow2(v) // vpl)
+        vpl = -(-v // x)
+        items = 2
     if mean_bag_len < 24:
         y = 1
     elif mean_bag_len < 96:

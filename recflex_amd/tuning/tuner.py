@@ -260,6 +260,9 @@ class Tuner:
             manager = TaskManager(list(range(max(1, tune_config.num_processes))))
             for key, build_dir in to_publish:
                 os.makedirs(build_dir, exist_ok=True)
+                stale = f"{build_dir}/librecom.so"      # a link to the cache from an earlier run:
+                if os.path.exists(stale):               # make would call it up to date
+                    os.remove(stale)
                 manager.add_task(compile_build, (build_dir,))
             manager.join()
         for key, build_dir in to_publish:
@@ -267,7 +270,9 @@ class Tuner:
             if not os.path.exists(lib):
                 raise Exception(f"build failed: {lib} was not produced")
             os.makedirs(os.path.dirname(self._cached_lib(key)), exist_ok=True)
-            shutil.copyfile(lib, self._cached_lib(key))
+            cached = self._cached_lib(key)
+            if not (os.path.exists(cached) and os.path.samefile(lib, cached)):
+                shutil.copyfile(lib, cached)
         for key, group in by_key.items():
             for output_dir, build_dir in group:
                 os.makedirs(build_dir, exist_ok=True)
