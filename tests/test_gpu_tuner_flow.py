@@ -89,10 +89,13 @@ def test_tournament_then_global_stage():
     cfg = prebuilt.fixture_tune_config(interference="model", remeasure=True, rounds=1, refine_passes=1)
     print("[case] tournament local stage", flush=True)
     res = tuner.tune(cfg)
-    for f in range(6):
-        for occ in cfg.occupancies:
-            assert len(res[f][occ]) == len(tuner.feat_sched_param_candidates[f])
-            assert np.isfinite(res[f][occ]).all() and min(res[f][occ]) > 0
+    for occ in cfg.occupancies:
+        admitted = tuner.admitted_candidates(occ)      # what the register census let in
+        for f in range(6):
+            t = np.asarray(res[f][occ])
+            assert len(t) == len(tuner.feat_sched_param_candidates[f]) and admitted[f]
+            assert np.isfinite(t[admitted[f]]).all() and t.min() > 0
+            assert np.isinf(np.delete(t, admitted[f])).all()
     picked = tuner.select_per_occupancy(res, cfg.occupancies)
     for i, occ in enumerate(cfg.occupancies):
         for f in range(6):
