@@ -318,13 +318,19 @@ extern "C" int recom_process(const recom_process_args *a) {
   const int xcd_segments = a->xcd_segments > 0 ? a->xcd_segments
                                                : (a->xcd_segments < 0 ? 0 : XCD_SEGMENTS);
 
-  hipLaunchKernelGGL(FusedKnl, dim3(grid), dim3(BLOCK_THREADS), st->dyn_lds,
-                     static_cast<hipStream_t>(a->stream),
-                     a->d_embed_table_ptrs, a->d_io_ptrs,
-                     static_cast<const char *>(a->d_arg_buffers), a->d_arg_buffer_offsets,
-                     a->d_output, a->batch, tile_bytes, xcd_segments, a->d_schedule_choice,
-                     a->d_times);
-  return static_cast<int>(hipGetLastError());
+  // hipLaunchKernel reports the error of this launch itself; the thread's last-error slot may
+  // still hold the failure of an unrelated earlier call and is not consulted
+  const char *arg_buffers = static_cast<const char *>(a->d_arg_buffers);
+  int batch = a->batch, tile_arg = tile_bytes, xcd_arg = xcd_segments;
+  void *kernel_args[] = {
+      const_cast<int64_t **>(&a->d_embed_table_ptrs), const_cast<int64_t **>(&a->d_io_ptrs),
+      &arg_buffers, const_cast<int64_t **>(&a->d_arg_buffer_offsets),
+      const_cast<float **>(&a->d_output), &batch, &tile_arg, &xcd_arg,
+      const_cast<int32_t **>(&a->d_schedule_choice),
+      const_cast<unsigned long long **>(&a->d_times)};
+  e = hipLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
+                      kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream));
+  return static_cast<int>(e);
 }
 '''
 

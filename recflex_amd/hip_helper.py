@@ -77,23 +77,32 @@ class HipInfoQuerier:
                 self.get_attribute(HIP_DEVICE_ATTRIBUTE_WALL_CLOCK_RATE, dev_ordinal))
 
 
+HIP_ERROR_NOT_SUPPORTED = 801
+
+
 class HipProfiler:
     """Range gate for an external profiler (hipProfilerStart/Stop).  rocprofv3 traces the whole
-    process and the tuner picks the kernel by name, so a runtime that ignores these calls
-    changes nothing."""
+    process and the tuner picks the kernel by name, so a runtime that does not implement these
+    calls (ROCm 7 answers hipErrorNotSupported) changes nothing: that answer is accepted, any
+    other error is raised as in the reference (RecFlex/cuda_helper.py CudaProfiler)."""
 
     def __init__(self):
         self._hip = _load_hip()
+        self.supported = True
+
+    def _call(self, name: str) -> None:
+        ret = getattr(self._hip, name)()
+        if ret == HIP_ERROR_NOT_SUPPORTED:
+            self.supported = False
+            self._hip.hipGetLastError()     # do not leave the refusal for the next caller to find
+        elif ret != 0:
+            raise Exception(f"{name}() returned {ret}")
 
     def start(self):
-        ret = self._hip.hipProfilerStart()
-        if ret != 0:
-            raise Exception(f"hipProfilerStart() returned {ret}")
+        self._call("hipProfilerStart")
 
     def stop(self):
-        ret = self._hip.hipProfilerStop()
-        if ret != 0:
-            raise Exception(f"hipProfilerStop() returned {ret}")
+        self._call("hipProfilerStop")
 
 
 # names of the reference module, for scripts written against it
