@@ -201,8 +201,10 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
     }
     if gather_floor:
         # the memory system's floor for this batch: the same rows fetched and dropped
+        from recflex_amd import gather_probe
         from recflex_amd.gather_probe import GatherProbe
         from recflex_amd.workloads import row_stride
+        gather_probe.build()            # compiles only if the library was not built ahead
         probe = GatherProbe(dev, tables, d_idx, [row_stride(f.dim, f.data_type) for f in wl.features])
         floor = probe.best_time_us(steps=min(steps, 10))
         res["gather_floor_us"] = floor["us"]
