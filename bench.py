@@ -23,7 +23,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0   # MI355X, HBM3E, published
-METRIC = "fused-kernel us + achieved HBM GB/s (% of MI355X peak) per model config"
+METRIC = "fused-kernel \u00b5s + achieved HBM GB/s (% of MI355X peak) per model config"
 
 # HBM bytes per launch (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, rocprofv3 --pmc, scale factors
 # from a 1 GiB copy in the same runs) of the tuned models, as recorded in
