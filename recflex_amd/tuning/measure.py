@@ -315,8 +315,9 @@ def measure_naive_candidate(ident: Tuple[int, int], data_npz: str, table_shape: 
 def _run_script_args(table_config_fname: str, build_dir: str, data_dir: str,
                      sample_batch_nums: int, spec_feat_id: Optional[int]) -> List[str]:
     script_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "run_script.py")
-    args = [sys.executable, script_path, "--table_config_fname", table_config_fname,
-            "--build_dir", build_dir, "--data_dir", data_dir,
+    # absolute paths: the profiler is started from /tmp, where it writes its scratch files
+    args = [sys.executable, script_path, "--table_config_fname", os.path.abspath(table_config_fname),
+            "--build_dir", os.path.abspath(build_dir), "--data_dir", os.path.abspath(data_dir),
             "--sample_batch_nums", str(sample_batch_nums)]
     if spec_feat_id is not None:
         args += ["--spec_feat_id", str(spec_feat_id)]
@@ -339,8 +340,10 @@ def rocprof_profile(table_config_fname: str, build_dir: str, data_dir: str, samp
     env = dict(os.environ)
     env["HIP_VISIBLE_DEVICES"] = str(gpu_id)
     env.setdefault("TMPDIR", "/tmp")
-    # like nsys in the reference, the profiler's own exit status is not trusted; the stats file is
-    subprocess.run(cmd, env=env, cwd="/tmp", stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    # like nsys in the reference, the profiler's own exit status is not trusted; the stats file
+    # is.  What the run printed is kept beside the report for the case that no file appears.
+    with open(f"{os.path.abspath(report_prefix)}.rocprofv3.log", "w") as log:
+        subprocess.run(cmd, env=env, cwd="/tmp", stdout=log, stderr=subprocess.STDOUT)
 
 
 # the reference's name for the global-stage worker

@@ -277,3 +277,15 @@ def test_build_climb_adopts_faster_production_builds(tmp_path, monkeypatch):
     # no trials: the start mix comes back with its own time
     mix0, t0 = t.build_climb(start, occ, scores, cfg._replace(build_climb_trials=0))
     assert mix0 == start and t0 == pytest.approx(sum(body_cost(x) for x in start))
+
+
+def test_profiler_command_uses_absolute_paths(tmp_path, monkeypatch):
+    """The global stage starts rocprofv3 from /tmp; a model directory given relative to the
+    caller's directory must still be found."""
+    from recflex_amd.tuning.measure import _run_script_args
+    monkeypatch.chdir(tmp_path)
+    args = _run_script_args("models/t/table_config.txt", "models/t/out/build", "models/t/data", 4, None)
+    for flag in ("--table_config_fname", "--build_dir", "--data_dir"):
+        value = args[args.index(flag) + 1]
+        assert os.path.isabs(value) and value.startswith(str(tmp_path))
+    assert os.path.isabs(args[1]) and args[1].endswith("run_script.py")
