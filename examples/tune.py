@@ -107,7 +107,8 @@ def create_tuner(args: argparse.Namespace) -> Tuner:
         output_dir = args.output_dir or os.path.join(ROOT, "recflex_amd", "_models", f"tune_{args.workload}")
         batches = [[] for _ in range(wl.num_features)]
         for k in range(args.workload_batches):
-            indices, offsets = gen_inputs(wl._replace(seed=wl.seed + 7919 * k))
+            # batches of the same distribution as the benchmark's, never the benchmark's own
+            indices, offsets = gen_inputs(wl._replace(seed=wl.seed + 7919 * (k + 1)))
             for f in range(wl.num_features):
                 batches[f].append((indices[f], offsets[f]))
         basic_config = BasicConfig(batch_sizes_fname="", data_fnames=[], schedule_config_fname="",
