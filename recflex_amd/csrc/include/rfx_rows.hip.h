@@ -72,6 +72,19 @@ template <int D> __device__ __forceinline__ f32x2 load_scale_bias(const char *__
 
 // acc[0..EPV) += decode(v).  For I8 only code*scale is added here; the bias is summed once per
 // lookup by the caller and added to every column after the bag is finished.
+#ifndef RFX_F16_FMA_MIX
+#define RFX_F16_FMA_MIX 1
+#endif
+
+// acc + (the fp16 value in the low (HI == 0) or high (HI == 1) half of w), rounded once
+template <int HI> __device__ __forceinline__ float add_half(float acc, uint32_t w) {
+  if constexpr (HI == 0)
+    asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel_hi:[1,0,0]" : "+v"(acc) : "v"(w));
+  else
+    asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(acc) : "v"(w));
+  return acc;
+}
+
 template <int DT, int VB>
 __device__ __forceinline__ void accumulate(float *acc, const Vec<VB> &v, float scale) {
   if constexpr (DT == F32) {
@@ -80,9 +93,16 @@ __device__ __forceinline__ void accumulate(float *acc, const Vec<VB> &v, float s
   } else if constexpr (DT == F16) {
 #pragma unroll
     for (int i = 0; i < VB / 4; ++i) {
+#if RFX_F16_FMA_MIX
+      // acc += half: one v_fma_mix_f32 (half * 1.0 + acc, the half taken straight from the low or
+      // high 16 bits of the loaded dword) instead of a conversion and an add; same rounding
+      acc[2 * i] = add_half<0>(acc[2 * i], v.w[i]);
+      acc[2 * i + 1] = add_half<1>(acc[2 * i + 1], v.w[i]);
+#else
       const f32x2 f = unpack_half2(v.w[i]);
       acc[2 * i] += f.x;
       acc[2 * i + 1] += f.y;
+#endif
     }
   } else {
 #pragma unroll
