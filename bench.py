@@ -71,7 +71,6 @@ def pick_model(name: str) -> str:
 def cpu_leg(wl, tables, indices, offsets, gpu_out, max_features: int):
     """Times the oracle on the host cores over a bounded sample (the first ``n`` features that
     keep the work near 10-30 s) and checks the GPU output of those features against it."""
-    import numpy as np
     import torch
     from oracle import oracle
     from recflex_amd.workloads import row_bytes

@@ -15,7 +15,6 @@ events instead of spawning rocprofv3.  The result is ``<output>/optimal/`` (sour
 """
 
 import argparse
-import json
 import multiprocessing as mp
 import os
 import sys

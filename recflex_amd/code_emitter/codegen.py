@@ -20,7 +20,7 @@ What is emitted is new:
 
 import json
 import os
-from typing import Any, Dict, List, NamedTuple, Optional, Tuple
+from typing import Any, Dict, List, NamedTuple, Tuple
 
 from .schedule_base import ScheduleBase, ScheduleVars, PreprocessVars
 from .build_basic import BasicBuilder

@@ -8,7 +8,7 @@ any number of emitted kernels can be used in one process.
 
 import ctypes
 import os
-from typing import List, Optional
+from typing import List
 
 _I32P = ctypes.POINTER(ctypes.c_int32)
 

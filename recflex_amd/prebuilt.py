@@ -18,7 +18,7 @@ its library is missing.  Names:
 
 import json
 import os
-from typing import Callable, Dict, List, NamedTuple, Optional, Tuple
+from typing import Callable, Dict, List, NamedTuple, Optional
 
 import numpy as np
 

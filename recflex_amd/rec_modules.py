@@ -20,7 +20,6 @@ accepted and ignored; tables may be fp32, fp16 or row-wise int8; the kernel runs
 current stream.  There is no CPU fallback: without a built library the modules raise.
 """
 
-from types import ModuleType
 from typing import List, Optional, Sequence, Tuple, Union
 
 import numpy as np
@@ -28,7 +27,7 @@ import torch
 import torch.nn as nn
 
 from .librecom import RecomLib
-from .quant import int8_row_stride, random_int8_table
+from .quant import random_int8_table
 
 _current_lib: Optional[RecomLib] = None
 

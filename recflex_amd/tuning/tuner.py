@@ -32,7 +32,7 @@ import numpy as np
 
 from recflex_amd.code_emitter import CodeEmitter, ScheduleBase, MetaData
 from recflex_amd.code_emitter.codegen import BAG_FIXED_BYTES, DEFAULT_TILE_BYTES, INDEX_BYTES
-from recflex_amd.utils import find_file, compile_build, os_check
+from recflex_amd.utils import compile_build, os_check
 from recflex_amd.task_manager import TaskManager
 from recflex_amd.parser import (parse_raw_data_batches, parse_table_shapes, parse_table_dtypes,
                                 parse_schedule_types, parse_knl_total_time)

@@ -6,12 +6,12 @@ import re
 
 import pytest
 
-from recflex_amd.code_emitter import CodeEmitter, MetaData, ScheduleBase, InputStats
+from recflex_amd.code_emitter import CodeEmitter, MetaData, ScheduleBase
 from recflex_amd.schedules import (SCHEDULE_MAPPING, BlockPerBagParams, BlockPerBagSchedule,
                                    SubWavefrontPerBagParams, SubWavefrontPerBagSchedule,
                                    ThreadPerBagSchedule, WavefrontPerBagParams,
                                    WavefrontPerBagSchedule, default_schedule, schedule_from_config)
-from recflex_amd.schedules.team import TeamParams, fits_registers
+from recflex_amd.schedules.team import fits_registers
 
 
 def test_metadata_row_formats():

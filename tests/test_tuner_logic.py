@@ -14,7 +14,7 @@ from recflex_amd.code_emitter import MetaData
 from recflex_amd.schedules import SCHEDULE_MAPPING, WarpPerSampleSchedule, OneHotSchedule
 from recflex_amd.tuning import BasicConfig, TuneConfig, Tuner
 from recflex_amd.tuning.tuner import padded_sched_num
-from recflex_amd.tuning.measure import load_batches, save_batches, tiles_per_feature
+from recflex_amd.tuning.measure import load_batches, tiles_per_feature
 
 
 def _tiny_tuner(tmp_path, feats=2, batches=2):
