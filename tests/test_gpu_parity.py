@@ -141,3 +141,47 @@ def test_pending_error_of_an_unrelated_call_does_not_fail_the_launch():
     prof.start()
     prof.stop()                      # accepted whether the runtime implements the gates or not
     assert not torch.isnan(torch.empty(4, device=dev).fill_(1.0)).any()    # nothing left pending
+
+
+@pytest.mark.parametrize("batch,seed", [(1, 0), (3, 1), (64, 2), (257, 3), (1000, 4)])
+def test_every_schedule_variant_on_ragged_batches(batch, seed):
+    """The 161-variant library (every template, lane split and element type) on batches it was
+    not built around: any batch size, bag lengths with a heavy tail, runs of empty bags, features
+    without a single lookup.  Integer-valued tables, so the comparison is bit for bit."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_tables
+
+    wl = prebuilt.model_spec("variants").workload
+    assert wl.table_values == "integer"
+    dev = torch.device("cuda", 0)
+    print(f"[case] variants on a ragged batch: B={batch} seed={seed}", flush=True)
+    rng = np.random.default_rng(1000 + seed)
+    tables = gen_tables(wl, dev)
+    indices, offsets = [], []
+    for f, spec in enumerate(wl.features):
+        kind = (f + seed) % 5
+        if kind == 0:
+            lens = np.zeros(batch, dtype=np.int64)                        # no lookup at all
+        elif kind == 1:
+            lens = rng.geometric(0.08, batch) * (rng.random(batch) < 0.6)  # heavy tail, 40 % empty
+        elif kind == 2:
+            lens = np.zeros(batch, dtype=np.int64)
+            lens[rng.integers(0, batch)] = 700                            # one long bag
+        elif kind == 3:
+            lens = rng.integers(0, 4, batch)
+        else:
+            lens = np.full(batch, 1 + f % 9)
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        indices.append(rng.integers(0, spec.rows, int(off[-1])).astype(np.int32))
+        offsets.append(off)
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib("variants"))
+    d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+    d_off = [torch.from_numpy(o).to(dev) for o in offsets]
+    got = layer.forward_indices(d_idx, d_off).cpu().numpy()
+    shrunk = wl._replace(batch=batch)
+    want = oracle_output(shrunk, [t.cpu().numpy() for t in tables], indices, offsets)
+    assert got.shape == want.shape == (batch, wl.embed_dim_sum)
+    bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+    assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
