@@ -179,7 +179,7 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
     float *__restrict__ {vars_.output},
     const int {vars_.embed_dim_offset},
     const int {vars_.bag_begin}, const int {vars_.bag_end},
-    char *__restrict__ {vars_.shmem}) {{
+    char *__restrict__ {vars_.shmem}, rfx::f32x4 *__restrict__ {vars_.stage}) {{
   {schedule.EmitScheduleBody(params)}
 }}
 '''
@@ -229,8 +229,11 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
   }}
 ''' if timing else ''
 
+        need_stage = self.out_vec() == 4 and any(flat[i][0].NeedsOutputStage(flat[i][1]) for i in body_ids)
+        stage_decl = (f"  __shared__ rfx::TeamStage<{vars_.BLOCK_THREADS}> s_stage;\n" if need_stage else "")
         call_args = (f"table, indices, offsets, d_output, embed_dim_offset, "
-                     f"{vars_.bag_begin}, {vars_.bag_end}, reinterpret_cast<char *>(&s)")
+                     f"{vars_.bag_begin}, {vars_.bag_end}, reinterpret_cast<char *>(&s), "
+                     + ("&s_stage.seg[0][0]" if need_stage else "nullptr"))
         cases = "".join(
             f"      case {feat_idx}: ProcessFeat{feat_idx}({call_args}); break;\n"
             for feat_idx in body_ids)
@@ -250,7 +253,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
   __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;
 
   __shared__ KnlTempStorage s;
-{timing_init}
+{stage_decl}{timing_init}
   const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
   const int total_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}>(
       s_bind, io, tile_bytes, c_lookup_bytes, c_bag_bytes, c_cand_begin, c_cand_gran,

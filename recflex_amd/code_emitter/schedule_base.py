@@ -91,6 +91,7 @@ class ScheduleVars(NamedTuple):
     """Names visible inside an emitted schedule body (reference: schedule_base.py:28-40)."""
     embed_table: str = "d_embed_table"       # const char *, base of this feature's table
     shmem: str = "s"                         # char *, the workgroup's LDS union
+    stage: str = "stage"                     # rfx::f32x4 *, LDS staging of team outputs (or null)
     indices: str = "d_indices"               # const int *, this feature's lookups
     offsets: str = "d_offsets"               # const int *, [batch + 1]
     output: str = "d_output"                 # float *, [batch, EMBED_DIM_SUM]
@@ -127,6 +128,10 @@ class ScheduleBase(ABC):
     @abstractmethod
     def EmitShmemType(self, params: NamedTuple) -> str:
         pass
+
+    def NeedsOutputStage(self, params: NamedTuple) -> bool:
+        """True if the body writes through the kernel's ``rfx::TeamStage`` LDS buffer."""
+        return False
 
     @abstractmethod
     def TileGranularity(self, params: NamedTuple) -> int:

@@ -23,6 +23,21 @@
 
 namespace rfx {
 
+// LDS staging of a team's output.  A lane of an fp16 (int8) team ends a bag with 8 (16)
+// consecutive output columns per row vector, i.e. 2 (4) float4 -- written straight from the
+// registers, each store instruction would put 16 bytes every 32 (64) bytes, four partial writes
+// per 128-byte line (measured: 3.6 TB/s against 4.9-6.1 TB/s for whole lines).  The team
+// therefore passes the segment through LDS and stores it with consecutive float4 per lane.
+// Every wavefront owns a fixed slice (the wavefronts of a workgroup drift apart and may be in
+// tiles of different features at the same time); fp32 teams never touch it.
+constexpr int kStageF4PerLane = 4;      // int8: 16 floats per lane and row vector
+#ifndef RFX_STAGE_MIN_F4
+#define RFX_STAGE_MIN_F4 2              // stage from this many float4 per lane and vector on
+#endif
+template <int BT> struct TeamStage {
+  f32x4 seg[BT / 64][64 * kStageF4PerLane];
+};
+
 // ---------------------------------------------------------------------------------------------
 // team_bags: teams of T <= 64 lanes; a workgroup of BT threads holds BT/T teams; team t sums
 // bags bag_begin + (t + k*TEAMS)*UB + [0, UB).
@@ -33,7 +48,8 @@ namespace rfx {
 // ---------------------------------------------------------------------------------------------
 template <int BT, int DT, int D, int X, int Y, int U, int UB, int VPP, int OVEC>
 __device__ __forceinline__ void
-team_bags(const char *__restrict__ table, const int *__restrict__ indices,
+team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
+          const int *__restrict__ indices,
           const int *__restrict__ offsets, float *__restrict__ out, const int esum,
           const int col_off, const int bag_begin, const int bag_end) {
   using R = Row<DT, D>;
@@ -202,7 +218,53 @@ team_bags(const char *__restrict__ table, const int *__restrict__ indices,
         }
       }
 
-      if (y == 0) {
+      if constexpr (OVEC == 4 && EPV / 4 >= RFX_STAGE_MIN_F4) {
+        // several float4 of consecutive columns per lane: through LDS, so that each store
+        // instruction of the team writes consecutive memory
+        constexpr int Q = EPV / 4;
+        static_assert(Q <= kStageF4PerLane, "stage slice too small");
+        // this team's part of its wavefront's slice
+        f32x4 *seg = stage + (tid >> 6) * (64 * kStageF4PerLane) + ((tid & 63) / T) * (X * Q);
+#pragma unroll
+        for (int i = 0; i < UB; ++i) {
+          const int bag = bag0 + i;
+          const bool live = y == 0 && bag < bag_end;
+          float *dst = out + static_cast<int64_t>(bag) * esum + col_off;
+#pragma unroll
+          for (int v = 0; v < VPP; ++v) {
+            if (v0 + v < VPL) {
+              const int first = (v0 + v) * X;                 // first row vector of the segment
+              const int nvec = R::V - first < X ? R::V - first : X;
+              if (live && x < nvec) {
+#pragma unroll
+                for (int q = 0; q < Q; ++q) {
+                  f32x4 t;
+                  t.x = acc[i][v][4 * q + 0]; t.y = acc[i][v][4 * q + 1];
+                  t.z = acc[i][v][4 * q + 2]; t.w = acc[i][v][4 * q + 3];
+                  if constexpr (DT == I8) t += bias_acc[i];
+                  seg[x * Q + q] = t;
+                }
+              }
+              // the lanes of a team sit in one wavefront: order its LDS writes before its reads
+              __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+              __builtin_amdgcn_wave_barrier();
+              __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+              if (live) {
+#pragma unroll
+                for (int k = 0; k < Q; ++k) {
+                  const int j = k * X + x;                    // float4 of the segment
+                  if (j < nvec * Q)
+                    *reinterpret_cast<f32x4 *>(dst + first * EPV + j * 4) = seg[j];
+                }
+              }
+              // ... and these reads before the next segment's writes
+              __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+              __builtin_amdgcn_wave_barrier();
+              __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            }
+          }
+        }
+      } else if (y == 0) {
 #pragma unroll
         for (int i = 0; i < UB; ++i) {
           const int bag = bag0 + i;
@@ -224,6 +286,7 @@ team_bags(const char *__restrict__ table, const int *__restrict__ indices,
       }
     }
   }
+  (void)stage;
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -109,12 +109,17 @@ class TeamScheduleBase(ScheduleBase):
         return f'''
   rfx::team_bags<{v.BLOCK_THREADS}, {m.dtype_id}, {m.embed_dim}, {p.lanes_x}, {p.lanes_y},
                  {p.items_per_thread}, {p.bags_per_team}, {p.vectors_per_pass}, {v.out_vec}>(
+      {v.stage},
       {v.embed_table}, {v.indices}, {v.offsets}, {v.output},
       {v.EMBED_DIM_SUM}, {v.embed_dim_offset}, {v.bag_begin}, {v.bag_end});
 '''
 
     def EmitShmemType(self, params: NamedTuple) -> str:
         return "char"
+
+    def NeedsOutputStage(self, params: NamedTuple) -> bool:
+        """fp16 / int8 teams stage their output through the kernel's ``TeamStage`` LDS buffer."""
+        return self.meta.elems_per_vector > 4
 
     def TileGranularity(self, params: NamedTuple) -> int:
         p = self.team_params(params)
