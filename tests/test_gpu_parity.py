@@ -185,3 +185,54 @@ def test_every_schedule_variant_on_ragged_batches(batch, seed):
     assert got.shape == want.shape == (batch, wl.embed_dim_sum)
     bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
     assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
+
+
+def test_launch_replays_inside_a_hip_graph():
+    """recom_process is a single kernel launch on the caller's stream (binding happens on the
+    device, no host-side task mapping, no copies), so a serving loop can capture it once and
+    replay it.  Captured after one eager call; replayed four times, each time with new bag
+    lengths and lookups written into the same index / offset buffers, with eager work and
+    synchronisations in between; every replay is compared bit for bit with an eager launch."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    wl = prebuilt.model_spec("c3s").workload
+    dev = torch.device("cuda", 0)
+    print(f"[case] c3s captured in a graph: F={wl.num_features} B={wl.batch}", flush=True)
+    tables = gen_tables(wl, dev)
+    batches = [gen_inputs(wl._replace(seed=wl.seed + 31 * k)) for k in range(4)]
+    capacity = [max(len(b[0][f]) for b in batches) for f in range(wl.num_features)]
+    d_idx = [torch.zeros(max(1, c), dtype=torch.int32, device=dev) for c in capacity]
+    d_off = [torch.zeros(wl.batch + 1, dtype=torch.int32, device=dev) for _ in range(wl.num_features)]
+    out = torch.empty(wl.batch, wl.embed_dim_sum, dtype=torch.float32, device=dev)
+    eager_out = torch.empty_like(out)
+
+    def load(batch):
+        indices, offsets = batch
+        for f in range(wl.num_features):
+            d_idx[f][:len(indices[f])].copy_(torch.from_numpy(indices[f]))
+            d_off[f].copy_(torch.from_numpy(offsets[f]))
+
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib("c3s"))
+    load(batches[0])
+    layer.forward_indices(d_idx, d_off, out=eager_out)       # first call: launch state, addresses
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        layer.forward_indices(d_idx, d_off, out=out)
+
+    for k in (1, 2, 3, 0):
+        load(batches[k])
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        layer.forward_indices(d_idx, d_off, out=eager_out)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int32), eager_out.view(torch.int32)), f"replay of batch {k}"
+        want = oracle_output(wl, [t.cpu().numpy() for t in tables], *batches[k])
+        _assert_parity(wl, got.cpu().numpy(), want)
