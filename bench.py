@@ -53,6 +53,8 @@ def parse_args():
                         "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     p.add_argument("--no-gather-floor", action="store_true",
                    help="skip the gather probe (bare fetch of the same rows, no sums, no output)")
+    p.add_argument("--no-torch-gpu", action="store_true",
+                   help="skip the unfused leg (one torch embedding_bag launch per feature on the GPU)")
     p.add_argument("--cpu-features", type=int, default=0,
                    help="bound the CPU leg to this many features (0 = choose from the size)")
     return p.parse_args()
@@ -126,9 +128,40 @@ def cpu_leg(wl, tables, indices, offsets, gpu_out, max_features: int):
     }, {"checked_features": n, "pass": bool(ok), "max_rel_err_beyond_atol": worst}
 
 
+def torch_gpu_leg(wl, tables, d_idx, d_off, steps: int, out) -> dict:
+    """The unfused way on the same GPU, for scale: one torch ``embedding_bag(sum)`` launch per
+    feature and a concatenation, timed with events over ``steps`` passes.  fp32 and fp16 tables
+    only (torch has no kernel for the int8 row format); its output is checked against the fused
+    kernel's."""
+    import torch
+    import torch.nn.functional as F
+
+    if any(f.data_type == "int8" for f in wl.features):
+        return {"skipped": "int8 rows have no torch embedding_bag"}
+
+    def one_pass():
+        cols = [F.embedding_bag(d_idx[f], tables[f], d_off[f], mode="sum", include_last_offset=True)
+                for f in range(wl.num_features)]
+        return torch.cat([c.float() for c in cols], dim=1)
+
+    got = one_pass()
+    torch.cuda.synchronize()
+    ref = out.view(wl.batch, wl.embed_dim_sum)
+    rtol = 1e-5 if wl.features[0].data_type == "float" else 2e-3     # torch accumulates fp16 in fp16
+    close = bool(torch.allclose(got, ref, rtol=rtol, atol=1e-5))
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        one_pass()
+    end.record()
+    torch.cuda.synchronize()
+    return {"us_per_pass": start.elapsed_time(end) * 1e3 / steps, "launches_per_pass": wl.num_features + 1,
+            "agrees_with_fused": close}
+
+
 def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: int,
                grid_blocks: int, cpu_features: int, xcd_segments: int = 0,
-               gather_floor: bool = True) -> dict:
+               gather_floor: bool = True, torch_gpu: bool = False) -> dict:
     import torch
     from recflex_amd import prebuilt
     from recflex_amd.rec_modules import FeatEmbed
@@ -210,6 +243,8 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
         res["gather_floor_setting"] = {k: v for k, v in floor.items() if k != "us"}
         res["kernel_over_gather_floor"] = kernel_us_avg / floor["us"]
         del probe
+    if torch_gpu:
+        res["torch_gpu_unfused"] = torch_gpu_leg(wl, tables, d_idx, d_off, min(steps, 20), out)
     if with_cpu:
         res["cpu_baseline"], res["check"] = cpu_leg(wl, tables, indices, offsets,
                                                     out, cpu_features)
@@ -241,7 +276,8 @@ def main():
 
     floor = not args.no_gather_floor
     head = run_config(args.workload, args.steps, args.warmup, not args.no_cpu, args.tile_bytes,
-                      args.grid_blocks, args.cpu_features, args.xcd_segments, floor)
+                      args.grid_blocks, args.cpu_features, args.xcd_segments, floor,
+                      torch_gpu=not args.no_torch_gpu)
     others = {}
     for name in [n for n in args.also.split(",") if n and n != args.workload]:
         try:
@@ -267,7 +303,7 @@ def main():
         "config": {"workload": f"{head['workload'].upper()}: {head['features']} features, batch "
                                f"{head['batch']}, sum(dim) {head['embed_dim_sum']}, "
                                f"{head['lookups']} lookups, {head['table_gb']} GB of tables",
-                   "model": head["model"], "bodies": head["bodies"],
+                   "build": head["model"], "bodies": head["bodies"],
                    "occupancy": head["occupancy"], "grid_blocks": head["grid_blocks"]},
         "kernel_us": head["kernel_us_avg"],
         "kernel_us_median": head["kernel_us_median"],
@@ -282,6 +318,8 @@ def main():
         # time of the bare fetch of the same rows (gather probe): what the memory system allows
         line["roofline"]["gather_floor_us"] = head["gather_floor_us"]
         line["roofline"]["kernel_over_gather_floor"] = head["kernel_over_gather_floor"]
+    if "torch_gpu_unfused" in head:
+        line["torch_gpu_unfused"] = head["torch_gpu_unfused"]
     if "cpu_baseline" in head:
         line["cpu_baseline"] = head["cpu_baseline"]
         line["check"] = head["check"]
