@@ -38,6 +38,20 @@ template <int BT> struct TeamStage {
   f32x4 seg[BT / 64][64 * kStageF4PerLane];
 };
 
+// threadIdx.x for a schedule body.  The fused kernel inlines some twenty bodies into one tile
+// loop; given the plain thread index the compiler computes every body's lane decomposition (team,
+// x, y and what follows from them) once before that loop and keeps all of it in registers
+// throughout: 128 registers and a spill for the 100-feature model, against 94 when each body
+// derives its values per tile.  The lane number therefore passes through an empty asm statement,
+// which nothing can be moved across.  The wavefront number stays a scalar and both ranges stay
+// visible to the compiler (the masks), which the straight-line paths of the bodies rely on.
+template <int BT> __device__ __forceinline__ int body_thread_id() {
+  static_assert(BT % 64 == 0 && ((BT / 64) & (BT / 64 - 1)) == 0, "1, 2, 4, 8 or 16 wavefronts");
+  int lane = threadIdx.x & 63;
+  asm volatile("" : "+v"(lane));
+  return (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) & (BT / 64 - 1)) * 64 + (lane & 63);
+}
+
 // ---------------------------------------------------------------------------------------------
 // team_bags: teams of T <= 64 lanes; a workgroup of BT threads holds BT/T teams; team t sums
 // bags bag_begin + (t + k*TEAMS)*UB + [0, UB).
@@ -62,7 +76,7 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
   constexpr int VB = R::VB;
   constexpr int EPV = R::EPV;
 
-  const int tid = threadIdx.x;
+  const int tid = body_thread_id<BT>();
   const int team = tid / T;
   const int lt = tid - team * T;
   const int y = lt / X;
@@ -321,7 +335,7 @@ block_bags(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ tab
   constexpr int EPV = R::EPV;
   constexpr int COLS = X * VPL * EPV;
 
-  const int tid = threadIdx.x;
+  const int tid = body_thread_id<BT>();
   const int y = tid / X;
   const int x = tid - y * X;
   const int wave = tid / 64;
