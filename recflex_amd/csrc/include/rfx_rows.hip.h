@@ -116,6 +116,14 @@ __device__ __forceinline__ void accumulate(float *acc, const Vec<VB> &v, float s
   }
 }
 
+// One store to the pooled output.  Output elements are written once and never read back by the
+// kernel; with the non-temporal hint they do not compete with the table rows for the L2
+// (measured against plain stores: 2-3 % less kernel time on the 100-, 200- and 400-feature
+// models, identical bits).
+template <typename T> __device__ __forceinline__ void store_streaming(T *p, const T v) {
+  __builtin_nontemporal_store(v, p);
+}
+
 // Store n fp32 values to the pooled output.  OVEC = widest store (in floats) the output
 // column offset of this feature allows: 4 -> global_store_dwordx4.
 template <int N, int OVEC>
@@ -124,17 +132,17 @@ __device__ __forceinline__ void store_floats(float *__restrict__ dst, const floa
 #pragma unroll
     for (int i = 0; i < N; i += 4) {
       f32x4 t; t.x = src[i]; t.y = src[i + 1]; t.z = src[i + 2]; t.w = src[i + 3];
-      *reinterpret_cast<f32x4 *>(dst + i) = t;
+      store_streaming(reinterpret_cast<f32x4 *>(dst + i), t);
     }
   } else if constexpr (OVEC >= 2 && N % 2 == 0) {
 #pragma unroll
     for (int i = 0; i < N; i += 2) {
       f32x2 t; t.x = src[i]; t.y = src[i + 1];
-      *reinterpret_cast<f32x2 *>(dst + i) = t;
+      store_streaming(reinterpret_cast<f32x2 *>(dst + i), t);
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < N; ++i) dst[i] = src[i];
+    for (int i = 0; i < N; ++i) store_streaming(dst + i, src[i]);
   }
 }
 

@@ -268,7 +268,7 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
                 for (int k = 0; k < Q; ++k) {
                   const int j = k * X + x;                    // float4 of the segment
                   if (j < nvec * Q)
-                    *reinterpret_cast<f32x4 *>(dst + first * EPV + j * 4) = seg[j];
+                    store_streaming(reinterpret_cast<f32x4 *>(dst + first * EPV + j * 4), seg[j]);
                 }
               }
               // ... and these reads before the next segment's writes
@@ -419,7 +419,7 @@ block_bags(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ tab
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) t += s.part_bias[w];
       }
-      dst[j] = t;
+      store_streaming(dst + j, t);
     }
   }
   (void)COLS;
