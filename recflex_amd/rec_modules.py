@@ -20,7 +20,7 @@ accepted and ignored; tables may be fp32, fp16 or row-wise int8; the kernel runs
 current stream.  There is no CPU fallback: without a built library the modules raise.
 """
 
-from typing import List, Optional, Sequence, Tuple, Union
+from typing import List, NamedTuple, Optional, Sequence, Tuple, Union
 
 import numpy as np
 import torch
@@ -128,7 +128,7 @@ class FeatEmbed(nn.Module):
 
         self.output_units = self.lib.embed_dim_sum
         self._io_cache_key = None
-        self._io_ptrs = None
+        self._io_bound = None
 
     def _check_tables(self) -> None:
         lib = self.lib
@@ -202,38 +202,64 @@ class FeatEmbed(nn.Module):
                             arg_buffers=arg_buffers.data_ptr(),
                             arg_buffer_offsets=data_buffer_offsets.data_ptr())
 
-    def forward_indices(self, indices: Sequence[torch.Tensor], offsets: Sequence[torch.Tensor],
+    def bind_inputs(self, indices: Sequence[torch.Tensor], offsets: Sequence[torch.Tensor]) -> "BoundInputs":
+        """Validate per-feature index / offset tensors once and upload their addresses.  The
+        result can be passed to ``forward_indices`` any number of times (the tensors may be
+        refilled in place between calls); a call with it costs no per-feature host work, which
+        for a model of a thousand features is 0.15 ms per call otherwise."""
+        n = len(self.embed_tables)
+        if len(indices) != n or len(offsets) != n:
+            raise ValueError(f"expected {n} index and offset tensors")
+        batch = offsets[0].numel() - 1
+        for f in range(n):
+            for name, t in (("indices", indices[f]), ("offsets", offsets[f])):
+                if t.dtype != torch.int32 or not t.is_contiguous() or t.device.type != "cuda":
+                    raise TypeError(f"{name}[{f}] must be a contiguous int32 device tensor")
+            if offsets[f].numel() != batch + 1:
+                raise ValueError("all features must share one batch size")
+        flat = [0] * (2 * n)
+        flat[0::2] = [t.data_ptr() for t in indices]
+        flat[1::2] = [t.data_ptr() for t in offsets]
+        io_ptrs = torch.tensor(flat, dtype=torch.int64, device=self.device)
+        return BoundInputs(batch, io_ptrs, (list(indices), list(offsets)))
+
+    def forward_indices(self, indices: Union["BoundInputs", Sequence[torch.Tensor]],
+                        offsets: Sequence[torch.Tensor] = None,
                         timing: bool = False, timing_schedules: int = None, tile_bytes: int = 0,
                         grid_blocks: int = 0, schedule_choice: torch.Tensor = None,
                         out: torch.Tensor = None, xcd_segments: int = 0):
         """Per-feature int32 device tensors ``indices[f]`` (``[L_f]``) and ``offsets[f]``
         (``[batch + 1]``, exclusive prefix sums, ``offsets[f][0] == 0``) -> ``[batch, sum(dim)]``
         fp32 (with ``timing=True``: ``(output, task_times)``).  ``out``: write into this
-        preallocated tensor instead of allocating one."""
-        n = len(self.embed_tables)
-        if len(indices) != n or len(offsets) != n:
-            raise ValueError(f"expected {n} index and offset tensors")
-        batch = offsets[0].numel() - 1
-        key = tuple(t.data_ptr() for t in indices) + tuple(t.data_ptr() for t in offsets) + (batch,)
-        if key != self._io_cache_key:
-            # new input tensors: validate them and upload their addresses
-            for f in range(n):
-                for name, t in (("indices", indices[f]), ("offsets", offsets[f])):
-                    if t.dtype != torch.int32 or not t.is_contiguous() or t.device.type != "cuda":
-                        raise TypeError(f"{name}[{f}] must be a contiguous int32 device tensor")
-                if offsets[f].numel() != batch + 1:
-                    raise ValueError("all features must share one batch size")
-            flat = [0] * (2 * n)
-            flat[0::2] = [t.data_ptr() for t in indices]
-            flat[1::2] = [t.data_ptr() for t in offsets]
-            self._io_ptrs = torch.tensor(flat, dtype=torch.int64, device=self.device)
-            self._io_cache_key = key
+        preallocated tensor instead of allocating one.  Instead of the two lists, the result of
+        ``bind_inputs`` may be given."""
+        if isinstance(indices, BoundInputs):
+            bound = indices
+        else:
+            n = len(self.embed_tables)
+            if offsets is None or len(indices) != n or len(offsets) != n:
+                raise ValueError(f"expected {n} index and offset tensors")
+            key = tuple(t.data_ptr() for t in indices) + tuple(t.data_ptr() for t in offsets) \
+                + (offsets[0].numel(),)
+            if key != self._io_cache_key:
+                # new input tensors: validate them and upload their addresses
+                self._io_bound = self.bind_inputs(indices, offsets)
+                self._io_cache_key = key
+            bound = self._io_bound
+        batch = bound.batch
         res = self._launch(batch, timing, timing_schedules, tile_bytes, grid_blocks,
                            schedule_choice=schedule_choice, out=out, xcd_segments=xcd_segments,
-                           io_ptrs=self._io_ptrs.data_ptr())
+                           io_ptrs=bound.io_ptrs.data_ptr())
         if timing:
             return res[0].view(batch, self.output_units), res[1]
         return res.view(batch, self.output_units)
+
+
+class BoundInputs(NamedTuple):
+    """Input tensors of ``FeatEmbed.forward_indices`` with their device address table."""
+    batch: int
+    io_ptrs: torch.Tensor       # int64 [2 * F] on the device: indices_f, offsets_f addresses
+    tensors: tuple              # keeps the bound tensors alive
 
 
 class FeatProcessEmbed(nn.Module):

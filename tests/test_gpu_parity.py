@@ -236,3 +236,37 @@ def test_launch_replays_inside_a_hip_graph():
         assert torch.equal(got.view(torch.int32), eager_out.view(torch.int32)), f"replay of batch {k}"
         want = oracle_output(wl, [t.cpu().numpy() for t in tables], *batches[k])
         _assert_parity(wl, got.cpu().numpy(), want)
+
+
+def test_bound_inputs_give_the_same_output():
+    """bind_inputs validates the tensors and uploads their addresses once; calls with its result
+    skip the per-feature host work and must launch exactly what the list form launches, also
+    after the bound tensors were refilled in place."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import BoundInputs, FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    wl = prebuilt.model_spec("c3s").workload
+    dev = torch.device("cuda", 0)
+    print(f"[case] c3s through bind_inputs: F={wl.num_features} B={wl.batch}", flush=True)
+    tables = gen_tables(wl, dev)
+    first, second = gen_inputs(wl), gen_inputs(wl._replace(seed=wl.seed + 5))
+    cap = [max(len(a), len(b), 1) for a, b in zip(first[0], second[0])]
+    d_idx = [torch.zeros(c, dtype=torch.int32, device=dev) for c in cap]
+    d_off = [torch.zeros(wl.batch + 1, dtype=torch.int32, device=dev) for _ in cap]
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib("c3s"))
+    bound = layer.bind_inputs(d_idx, d_off)
+    assert isinstance(bound, BoundInputs) and bound.batch == wl.batch
+    for indices, offsets in (first, second):
+        for f in range(wl.num_features):
+            d_idx[f][:len(indices[f])].copy_(torch.from_numpy(indices[f]))
+            d_off[f].copy_(torch.from_numpy(offsets[f]))
+        got = layer.forward_indices(bound).cpu().numpy()
+        same = layer.forward_indices(d_idx, d_off).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), same.view(np.uint32))
+        _assert_parity(wl, got, oracle_output(wl, [t.cpu().numpy() for t in tables], indices, offsets))
+    with pytest.raises(TypeError):
+        layer.bind_inputs([t.long() for t in d_idx], d_off)
+    with pytest.raises(ValueError):
+        layer.bind_inputs(d_idx[:-1], d_off[:-1])
