@@ -117,6 +117,21 @@ def _edge() -> ModelSpec:
     return ModelSpec(wl, fs, None)      # no occupancy: natural register use, no LDS pad
 
 
+def _other_block_size(block_threads: int) -> ModelSpec:
+    """Every element type and template at a workgroup size other than 256 (``tune.py -b``)."""
+    combos = [("float", 8, 3.0), ("float", 32, 40.0), ("float", 128, 1.0), ("half", 64, 25.0),
+              ("half", 256, 2.0), ("int8", 32, 9.0), ("int8", 128, 60.0), ("float", 64, 900.0)]
+    feats = [FeatureSpec(400 + 31 * i, d, t, m, False, 0.1, 1.0) for i, (t, d, m) in enumerate(combos)]
+    wl = Workload(f"b{block_threads}", 150, 515 + block_threads, tuple(feats), "integer")
+    fs = default_feat_schedules(metas_of(wl), [expected_bag_len(f) for f in feats], block_threads)
+    # the default rules pick sub-wavefront teams throughout: put the other templates in by hand
+    for f, cls in ((0, ThreadPerBagSchedule), (1, WavefrontPerBagSchedule), (3, WavefrontPerBagSchedule),
+                   (len(feats) - 1, BlockPerBagSchedule)):
+        sched = cls(MetaData(feats[f].dim, feats[f].data_type), block_threads)
+        fs[f] = (sched, sched.GenParamCandidates()[0])
+    return ModelSpec(wl, fs, None)
+
+
 _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c1": lambda: _default(make_workload("C1")),
     "c2": lambda: _default(make_workload("C2")),
@@ -134,6 +149,8 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c5s": lambda: _default(make_workload("C5", batch=256, num_features=24, max_rows=50_000)),
     "variants": _variants,
     "edge": _edge,
+    "b128": lambda: _other_block_size(128),
+    "b512": lambda: _other_block_size(512),
 }
 
 

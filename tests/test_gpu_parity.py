@@ -78,6 +78,15 @@ def test_integer_tables_are_bit_exact(name):
     assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
 
 
+@pytest.mark.parametrize("name", ["b128", "b512"])
+def test_other_workgroup_sizes_are_bit_exact(name):
+    """Libraries emitted for 128 and 512 threads per workgroup (2 and 8 wavefronts): every
+    template and element type, integer-valued tables, identical bits."""
+    wl, got, want = _run_model(name)
+    bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+    assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
+
+
 def test_onehot_is_bit_exact():
     """Bags of exactly one lookup are a row copy: identical bits (C2 shape, shrunk)."""
     wl, got, want = _run_model("c2s")
