@@ -57,7 +57,7 @@ typedef struct recom_info {
   int32_t reserved[5];
 } recom_info;
 
-#define RECOM_ABI_VERSION 1
+#define RECOM_ABI_VERSION 2
 
 /* Static description of the emitted kernel.  No reference counterpart as a function: the
  * reference bakes the same numbers into process.cu (EMBED_DIM_SUM, block_threads,
@@ -135,6 +135,12 @@ typedef struct recom_process_args {
   unsigned long long *d_times;
   /* hipStream_t to launch on (NULL = the null stream) */
   void *stream;
+  /* floats between the starts of consecutive output rows; 0 = embed_dim_sum (a dense
+   * [batch, embed_dim_sum] output, the only form the reference has).  A larger stride lets
+   * several libraries -- a model split by features over libraries or GPUs -- write their column
+   * slabs into one [batch, sum of all] buffer.  Must be a multiple of 4 when embed_dim_sum is
+   * (the kernel then stores 16 bytes at a time), and d_output aligned likewise. */
+  int64_t output_row_stride;
 } recom_process_args;
 
 /* Launch the fused kernel: for every feature f and sample b,

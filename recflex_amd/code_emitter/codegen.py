@@ -177,7 +177,7 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
     const int *__restrict__ {vars_.indices},
     const int *__restrict__ {vars_.offsets},
     float *__restrict__ {vars_.output},
-    const int {vars_.embed_dim_offset},
+    const int {vars_.out_row_stride}, const int {vars_.embed_dim_offset},
     const int {vars_.bag_begin}, const int {vars_.bag_end},
     char *__restrict__ {vars_.shmem}, rfx::f32x4 *__restrict__ {vars_.stage}) {{
   {schedule.EmitScheduleBody(params)}
@@ -231,7 +231,7 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
 
         need_stage = self.out_vec() == 4 and any(flat[i][0].NeedsOutputStage(flat[i][1]) for i in body_ids)
         stage_decl = (f"  __shared__ rfx::TeamStage<{vars_.BLOCK_THREADS}> s_stage;\n" if need_stage else "")
-        call_args = (f"table, indices, offsets, d_output, embed_dim_offset, "
+        call_args = (f"table, indices, offsets, d_output, {vars_.out_row_stride}, embed_dim_offset, "
                      f"{vars_.bag_begin}, {vars_.bag_end}, reinterpret_cast<char *>(&s), "
                      + ("&s_stage.seg[0][0]" if need_stage else "nullptr"))
         cases = "".join(
@@ -249,7 +249,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     float *__restrict__ d_output,
     const int batch, const int tile_bytes, const int xcd_segments,
     const int *__restrict__ d_schedule_choice,
-    unsigned long long *__restrict__ d_times) {{
+    unsigned long long *__restrict__ d_times, const int {vars_.out_row_stride}) {{
   __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;
 
   __shared__ KnlTempStorage s;
@@ -310,6 +310,11 @@ extern "C" int recom_process(const recom_process_args *a) {
   if (!TIMING && a->d_times) return static_cast<int>(hipErrorInvalidValue);
   if (a->tile_bytes < 0 || a->grid_blocks < 0 || a->xcd_segments > 4096)
     return static_cast<int>(hipErrorInvalidValue);
+  // the output: dense rows unless a stride is given; aligned for the widest store of the kernel
+  const int64_t row_stride = a->output_row_stride ? a->output_row_stride : EMBED_DIM_SUM;
+  if (row_stride < EMBED_DIM_SUM || row_stride > 0x7fffffff || row_stride % OUT_VEC != 0 ||
+      reinterpret_cast<uintptr_t>(a->d_output) % (OUT_VEC * sizeof(float)) != 0)
+    return static_cast<int>(hipErrorInvalidValue);
   if (a->batch == 0) return static_cast<int>(hipSuccess);
 
   const rfx::LaunchState *st = nullptr;
@@ -325,12 +330,13 @@ extern "C" int recom_process(const recom_process_args *a) {
   // still hold the failure of an unrelated earlier call and is not consulted
   const char *arg_buffers = static_cast<const char *>(a->d_arg_buffers);
   int batch = a->batch, tile_arg = tile_bytes, xcd_arg = xcd_segments;
+  int stride_arg = static_cast<int>(row_stride);
   void *kernel_args[] = {
       const_cast<int64_t **>(&a->d_embed_table_ptrs), const_cast<int64_t **>(&a->d_io_ptrs),
       &arg_buffers, const_cast<int64_t **>(&a->d_arg_buffer_offsets),
       const_cast<float **>(&a->d_output), &batch, &tile_arg, &xcd_arg,
       const_cast<int32_t **>(&a->d_schedule_choice),
-      const_cast<unsigned long long **>(&a->d_times)};
+      const_cast<unsigned long long **>(&a->d_times), &stride_arg};
   e = hipLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
                       kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream));
   return static_cast<int>(e);

@@ -97,6 +97,7 @@ class ScheduleVars(NamedTuple):
     output: str = "d_output"                 # float *, [batch, EMBED_DIM_SUM]
     embed_dim_offset: str = "embed_dim_offset"
     EMBED_DIM_SUM: str = "EMBED_DIM_SUM"
+    out_row_stride: str = "out_row_stride"   # floats between output rows (EMBED_DIM_SUM if dense)
     BLOCK_THREADS: str = "BLOCK_THREADS"
     bag_begin: str = "bag_begin"             # this tile sums bags [bag_begin, bag_end)
     bag_end: str = "bag_end"

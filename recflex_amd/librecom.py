@@ -53,10 +53,11 @@ class RecomProcessArgs(ctypes.Structure):
         ("d_schedule_choice", ctypes.c_void_p),
         ("d_times", ctypes.c_void_p),
         ("stream", ctypes.c_void_p),
+        ("output_row_stride", ctypes.c_int64),
     ]
 
 
-RECOM_ABI_VERSION = 1
+RECOM_ABI_VERSION = 2
 EXPORTED_SYMBOLS = ("recom_get_info", "recom_get_feature_tables", "recom_get_candidate_counts",
                     "recom_get_launch_info",
                     "recom_get_max_concurrent_blocks", "recom_process")
@@ -137,12 +138,12 @@ class RecomLib:
     def process(self, table_ptrs: int, output: int, batch: int, *, io_ptrs: int = 0,
                 arg_buffers: int = 0, arg_buffer_offsets: int = 0, tile_bytes: int = 0,
                 grid_blocks: int = 0, xcd_segments: int = 0, schedule_choice: int = 0,
-                times: int = 0, stream: int = 0) -> None:
+                times: int = 0, stream: int = 0, output_row_stride: int = 0) -> None:
         """All pointer arguments are raw device addresses (``tensor.data_ptr()``)."""
         args = RecomProcessArgs(table_ptrs or None, io_ptrs or None, arg_buffers or None,
                                 arg_buffer_offsets or None, output or None, batch, tile_bytes,
                                 grid_blocks, xcd_segments, schedule_choice or None, times or None,
-                                stream or None)
+                                stream or None, output_row_stride)
         rc = self.lib.recom_process(ctypes.byref(args))
         if rc != 0:
             raise RecomError("recom_process", rc)

@@ -152,12 +152,20 @@ class FeatEmbed(nn.Module):
     def _launch(self, batch: int, timing: bool, timing_schedules: Optional[int], tile_bytes: int,
                 grid_blocks: int, schedule_choice: torch.Tensor = None, out: torch.Tensor = None,
                 xcd_segments: int = 0, **inputs):
+        row_stride = 0
         if out is not None:
             if out.dtype != torch.float32 or out.numel() != batch * self.output_units \
-                    or not out.is_contiguous() or out.device.type != "cuda":
-                raise TypeError(f"out must be a contiguous fp32 device tensor of "
+                    or out.device.type != "cuda":
+                raise TypeError(f"out must be an fp32 device tensor of "
                                 f"{batch * self.output_units} elements")
-            output = out.view(-1)
+            if out.is_contiguous():
+                output = out.view(-1)
+            elif out.dim() == 2 and out.shape == (batch, self.output_units) and out.stride(1) == 1:
+                # a column slab of a wider buffer: the library writes rows out.stride(0) apart
+                output, row_stride = out, out.stride(0)
+            else:
+                raise TypeError("out must be contiguous, or a [batch, sum(dim)] view with unit "
+                                "column stride (a column slab of a wider buffer)")
         else:
             output = torch.empty([batch * self.output_units], dtype=torch.float32, device=self.device)
         times = None
@@ -173,7 +181,8 @@ class FeatEmbed(nn.Module):
         stream = torch.cuda.current_stream(self.device).cuda_stream
         self.lib.process(self.embed_table_ptrs.data_ptr(), output.data_ptr(), batch,
                          tile_bytes=tile_bytes, grid_blocks=grid_blocks, xcd_segments=xcd_segments,
-                         times=times.data_ptr() if times is not None else 0, stream=stream, **inputs)
+                         times=times.data_ptr() if times is not None else 0, stream=stream,
+                         output_row_stride=row_stride, **inputs)
         if timing:
             n = len(self.embed_tables)
             if not timing_schedules or timing_schedules > n:

@@ -47,7 +47,7 @@ class BlockPerBagSchedule(ScheduleBase):
                   {params.items_per_thread}, {params.chunk}>(
       *reinterpret_cast<{self._storage(params)} *>({v.shmem}),
       {v.embed_table}, {v.indices}, {v.offsets}, {v.output},
-      {v.EMBED_DIM_SUM}, {v.embed_dim_offset}, {v.bag_begin}, {v.bag_end});
+      {v.out_row_stride}, {v.embed_dim_offset}, {v.bag_begin}, {v.bag_end});
 '''
 
     def EmitShmemType(self, params: BlockPerBagParams) -> str:

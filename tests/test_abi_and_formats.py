@@ -54,9 +54,10 @@ def test_host_library_exports_every_host_symbol():
 
 def test_ctypes_structs_match_header_layout():
     # recom_info: 11 named int32 + 5 reserved; recom_process_args: 5 pointers, 4 int32,
-    # 3 pointers on LP64
+    # 3 pointers and an int64 on LP64
     assert ctypes.sizeof(RecomInfo) == 16 * 4
-    assert ctypes.sizeof(RecomProcessArgs) == 5 * 8 + 4 * 4 + 3 * 8
+    assert ctypes.sizeof(RecomProcessArgs) == 5 * 8 + 4 * 4 + 3 * 8 + 8
+    assert RecomProcessArgs.output_row_stride.offset == 80
     assert RecomProcessArgs.batch.offset == 40 and RecomProcessArgs.d_schedule_choice.offset == 56
     assert RecomProcessArgs.d_times.offset == 64
     src = open(HEADER).read()
@@ -81,8 +82,19 @@ def test_process_rejects_bad_arguments_without_a_device():
     assert r.lib.recom_process(ctypes.byref(a)) == 1
     a = RecomProcessArgs(d_embed_table_ptrs=8, d_io_ptrs=8, d_output=8, batch=4, d_times=8)
     assert r.lib.recom_process(ctypes.byref(a)) == 1         # timers on a non-timing build
-    a = RecomProcessArgs(d_embed_table_ptrs=8, d_io_ptrs=8, d_output=8, batch=0)
+    a = RecomProcessArgs(d_embed_table_ptrs=8, d_io_ptrs=8, d_output=16, batch=0)
     assert r.lib.recom_process(ctypes.byref(a)) == 0         # empty batch: nothing to launch
+    # output rows: a stride below the row length, one that breaks the 16-byte stores of a
+    # library whose sum of dims is a multiple of 4, a misaligned base
+    assert r.embed_dim_sum % 4 == 0
+    for bad in ({"output_row_stride": r.embed_dim_sum - 4}, {"output_row_stride": r.embed_dim_sum + 2},
+                {"d_output": 24}):
+        kw = dict(d_embed_table_ptrs=8, d_io_ptrs=8, d_output=16, batch=0)
+        kw.update(bad)
+        assert r.lib.recom_process(ctypes.byref(RecomProcessArgs(**kw))) == 1, bad
+    a = RecomProcessArgs(d_embed_table_ptrs=8, d_io_ptrs=8, d_output=16, batch=0,
+                         output_row_stride=r.embed_dim_sum + 64)
+    assert r.lib.recom_process(ctypes.byref(a)) == 0
 
 
 def test_missing_library_fails_loudly():

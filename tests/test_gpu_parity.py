@@ -279,3 +279,47 @@ def test_bound_inputs_give_the_same_output():
         layer.bind_inputs([t.long() for t in d_idx], d_off)
     with pytest.raises(ValueError):
         layer.bind_inputs(d_idx[:-1], d_off[:-1])
+
+
+def test_two_libraries_write_column_slabs_of_one_buffer():
+    """output_row_stride: a model split by features over two libraries (or GPUs) writes each
+    library's [batch, sum(dim)] block straight into its columns of the common output."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    dev = torch.device("cuda", 0)
+    parts = []
+    for name in ("c3s", "c5s"):
+        wl = prebuilt.model_spec(name).workload._replace(batch=100)
+        tables = gen_tables(wl, dev)
+        indices, offsets = gen_inputs(wl)
+        parts.append((name, wl, tables, indices, offsets))
+    widths = [p[1].embed_dim_sum for p in parts]
+    print(f"[case] slabs of {widths} columns in one [100, {sum(widths) + 8}] buffer", flush=True)
+    whole = torch.full((100, sum(widths) + 8), float("nan"), dtype=torch.float32, device=dev)
+    col = 4                                     # slabs need not start at column 0
+    for (name, wl, tables, indices, offsets), width in zip(parts, widths):
+        layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib(name))
+        d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+        d_off = [torch.from_numpy(o).to(dev) for o in offsets]
+        got = layer.forward_indices(d_idx, d_off, out=whole[:, col:col + width])
+        assert got.data_ptr() == whole[:, col:col + width].data_ptr()
+        col += width
+    torch.cuda.synchronize()
+    host = whole.cpu().numpy()
+    assert np.isnan(host[:, :4]).all() and np.isnan(host[:, col:]).all()    # nothing outside the slabs
+    col = 4
+    for (name, wl, tables, indices, offsets), width in zip(parts, widths):
+        want = oracle_output(wl, [t.cpu().numpy() for t in tables], indices, offsets)
+        _assert_parity(wl, np.ascontiguousarray(host[:, col:col + width]), want)
+        col += width
+    # a slab whose columns would break the kernel's 16-byte stores is refused
+    from recflex_amd.librecom import RecomError
+    name, wl, tables, indices, offsets = parts[0]
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib(name))
+    d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+    d_off = [torch.from_numpy(o).to(dev) for o in offsets]
+    with pytest.raises(RecomError):
+        layer.forward_indices(d_idx, d_off, out=whole[:, 2:2 + widths[0]])
