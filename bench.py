@@ -242,6 +242,10 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
         res["gather_floor_us"] = floor["us"]
         res["gather_floor_setting"] = {k: v for k, v in floor.items() if k != "us"}
         res["kernel_over_gather_floor"] = kernel_us_avg / floor["us"]
+        # ... and the same rows fetched plus an output of this size written as whole cache lines
+        with_output = probe.time_with_output_us(floor, outbuf, steps=min(steps, 10))
+        res["gather_write_floor_us"] = with_output
+        res["kernel_over_gather_write_floor"] = kernel_us_avg / with_output
         del probe
     if torch_gpu:
         res["torch_gpu_unfused"] = torch_gpu_leg(wl, tables, d_idx, d_off, min(steps, 20), out)
@@ -318,6 +322,9 @@ def main():
         # time of the bare fetch of the same rows (gather probe): what the memory system allows
         line["roofline"]["gather_floor_us"] = head["gather_floor_us"]
         line["roofline"]["kernel_over_gather_floor"] = head["kernel_over_gather_floor"]
+        # the gather plus the writing of an output of this size (whole lines, once)
+        line["roofline"]["gather_write_floor_us"] = head["gather_write_floor_us"]
+        line["roofline"]["kernel_over_gather_write_floor"] = head["kernel_over_gather_write_floor"]
     if "torch_gpu_unfused" in head:
         line["torch_gpu_unfused"] = head["torch_gpu_unfused"]
     if "cpu_baseline" in head:

@@ -1,7 +1,10 @@
 // Gather probe: reads exactly the table rows a batch looks up -- same tables, same index
 // streams, 16-byte loads -- and does nothing else (no bags, no sums, no output).  Its run time is
 // the floor the memory system sets for any kernel that has to fetch those rows, hot rows served
-// by the caches included; bench.py reports the fused kernel's time beside it.
+// by the caches included; bench.py reports the fused kernel's time beside it.  On request it
+// also writes as many bytes as the pooled output has, in the friendliest way there is (each
+// wavefront stores a contiguous run of whole cache lines after each chunk of lookups): the
+// floor for fetching the rows and writing an output of that size.
 //
 // No counterpart in the reference.  Measurement aid only: the product path never calls it.
 #include <hip/hip_runtime.h>
@@ -34,7 +37,7 @@ __global__ void __launch_bounds__(256)
 gather_probe_knl(const Chunk *__restrict__ chunks, const int n_chunks, const int segments,
                  const int64_t *__restrict__ table_ptrs, const int64_t *__restrict__ index_ptrs,
                  const int32_t *__restrict__ row_strides, const int32_t *__restrict__ row_vectors,
-                 float *__restrict__ sink) {
+                 float *__restrict__ sink, f32x4 *__restrict__ out, const int64_t out_f4) {
   const int lane = threadIdx.x & 63;
   const int wave_in_wg = threadIdx.x >> 6;
   const int groups = (n_chunks + 3) / 4;              // a workgroup takes four chunks at a time
@@ -84,6 +87,13 @@ gather_probe_knl(const Chunk *__restrict__ chunks, const int n_chunks, const int
         for (int u = 0; u < U; ++u) acc += buf[u];
       }
     }
+    if (out_f4 > 0) {
+      // this chunk's share of the output-sized buffer
+      const int64_t per = (out_f4 + n_chunks - 1) / n_chunks;
+      const int64_t lo = c * per;
+      const int64_t hi = lo + per < out_f4 ? lo + per : out_f4;
+      for (int64_t i = lo + lane; i < hi; i += 64) __builtin_nontemporal_store(acc, out + i);
+    }
   }
   // keeps the loads alive; never true for finite table values
   if (acc.x + acc.y + acc.z + acc.w == 1.2345e38f) sink[threadIdx.x] = acc.x;
@@ -95,30 +105,36 @@ gather_probe_knl(const Chunk *__restrict__ chunks, const int n_chunks, const int
 // {int32 feat, begin, count, log2x}; table_ptrs / index_ptrs: device int64[F]; row_strides /
 // row_vectors: device int32[F] (bytes between rows, 16-byte vectors per row); sink: device
 // float[256]; in_flight: 2, 4 or 8 row loads per lane; segments: chunk-space segments per XCD
-// (0 = flat).  Returns the hipError_t of the launch.
+// (0 = flat); out / out_bytes: device buffer (16-byte aligned) that is written once, spread over
+// the chunks, or NULL / 0 for the bare gather.  Returns the hipError_t of the launch.
 extern "C" int gather_probe_launch(const void *chunks, int n_chunks, const int64_t *table_ptrs,
                                    const int64_t *index_ptrs, const int32_t *row_strides,
                                    const int32_t *row_vectors, float *sink, int grid_blocks,
-                                   int in_flight, int segments, void *stream) {
+                                   int in_flight, int segments, void *stream, void *out,
+                                   int64_t out_bytes) {
   if (!chunks || !table_ptrs || !index_ptrs || !row_strides || !row_vectors || !sink ||
       n_chunks < 0 || grid_blocks <= 0 || segments < 0)
     return static_cast<int>(hipErrorInvalidValue);
+  if ((out_bytes > 0 && !out) || out_bytes < 0 || reinterpret_cast<uintptr_t>(out) % 16 != 0)
+    return static_cast<int>(hipErrorInvalidValue);
   if (n_chunks == 0) return 0;
+  f32x4 *out4 = static_cast<f32x4 *>(out);
+  const int64_t out_f4 = out_bytes / 16;
   const dim3 grid(grid_blocks), block(256);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const Chunk *ch = static_cast<const Chunk *>(chunks);
   switch (in_flight) {
   case 2:
     hipLaunchKernelGGL(gather_probe_knl<2>, grid, block, 0, s, ch, n_chunks, segments, table_ptrs,
-                       index_ptrs, row_strides, row_vectors, sink);
+                       index_ptrs, row_strides, row_vectors, sink, out4, out_f4);
     break;
   case 4:
     hipLaunchKernelGGL(gather_probe_knl<4>, grid, block, 0, s, ch, n_chunks, segments, table_ptrs,
-                       index_ptrs, row_strides, row_vectors, sink);
+                       index_ptrs, row_strides, row_vectors, sink, out4, out_f4);
     break;
   case 8:
     hipLaunchKernelGGL(gather_probe_knl<8>, grid, block, 0, s, ch, n_chunks, segments, table_ptrs,
-                       index_ptrs, row_strides, row_vectors, sink);
+                       index_ptrs, row_strides, row_vectors, sink, out4, out_f4);
     break;
   default:
     return static_cast<int>(hipErrorInvalidValue);

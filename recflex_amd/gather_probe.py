@@ -61,7 +61,8 @@ class GatherProbe:
         self.lib = ctypes.CDLL(path)
         self.lib.gather_probe_launch.restype = ctypes.c_int
         self.lib.gather_probe_launch.argtypes = [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 5 + \
-                                                [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+                                                [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                                 ctypes.c_void_p, ctypes.c_int64]
         self.device = device
         self.tables, self.d_indices = tables, d_indices          # kept alive
         self.num_lookups = [int(i.numel()) for i in d_indices]
@@ -85,13 +86,18 @@ class GatherProbe:
         self.d_chunks = torch.from_numpy(chunks).to(self.device) if len(chunks) else \
             torch.zeros((1, 4), dtype=torch.int32, device=self.device)
 
-    def launch(self, in_flight: int = 4, workgroups_per_cu: int = 8, segments: int = 0) -> None:
+    def launch(self, in_flight: int = 4, workgroups_per_cu: int = 8, segments: int = 0,
+               out=None) -> None:
+        """``out``: a device tensor the probe also fills once (whole cache lines, spread over the
+        run): the gather plus the writing of an output of that size."""
         import torch
         rc = self.lib.gather_probe_launch(self.d_chunks.data_ptr(), self.n_chunks, self.d_tables.data_ptr(),
                                           self.d_index_ptrs.data_ptr(), self.d_strides.data_ptr(),
                                           self.d_vectors.data_ptr(), self.d_sink.data_ptr(),
                                           self.cus * workgroups_per_cu, in_flight, segments,
-                                          torch.cuda.current_stream(self.device).cuda_stream)
+                                          torch.cuda.current_stream(self.device).cuda_stream,
+                                          out.data_ptr() if out is not None else None,
+                                          out.numel() * out.element_size() if out is not None else 0)
         if rc:
             raise RuntimeError(f"gather_probe_launch: hipError_t {rc}")
 
@@ -125,3 +131,11 @@ class GatherProbe:
                             best = {"us": t, "in_flight": u, "workgroups_per_cu": occ,
                                     "segments": seg, "chunk_bytes": chunk}
         return best
+
+    def time_with_output_us(self, setting: dict, out, steps: int = 10) -> float:
+        """The probe at ``setting`` (a result of ``best_time_us``) when it also fills ``out``
+        once per launch: rows fetched and an output of that size written."""
+        self.set_chunks(chunk_bytes=setting["chunk_bytes"])
+        return self.time_us(steps=steps, in_flight=setting["in_flight"],
+                            workgroups_per_cu=setting["workgroups_per_cu"],
+                            segments=setting["segments"], out=out)

@@ -114,6 +114,14 @@ def test_gather_probe_runs():
         assert probe.time_us(steps=3, warmup=1, **kwargs) > 0
     best = probe.best_time_us(steps=2)
     assert best["us"] > 0 and best["in_flight"] in (2, 4, 8)
+    # with an output-sized buffer to fill: every byte of it is written, nothing beyond it
+    # (what is written are sums of raw table bits read as floats, possibly NaN: compare bits)
+    mark = 0x4B1D4B1D
+    buf = torch.full((wl.batch * wl.embed_dim_sum + 8,), mark, dtype=torch.int32, device=dev)
+    assert probe.time_with_output_us(best, buf[4:-4].view(torch.float32), steps=2) > 0
+    torch.cuda.synchronize()
+    host = buf.cpu().numpy()
+    assert (host[:4] == mark).all() and (host[-4:] == mark).all() and (host[4:-4] != mark).all()
 
 
 def test_pending_error_of_an_unrelated_call_does_not_fail_the_launch():
