@@ -50,7 +50,8 @@ typedef struct recom_info {
   int32_t occupancy;      /* workgroups per CU the kernel was emitted for (0 = not limited) */
   int32_t num_bodies;     /* distinct schedule bodies after de-duplication */
   int32_t timing;         /* 1 if built with per-feature device timers */
-  int32_t tile_bytes;     /* default memory traffic per tile used by the run-time binding */
+  int32_t tile_bytes;     /* default memory traffic per tile of the run-time binding; 0 = chosen
+                           * per batch on the device from the batch's total traffic */
   int32_t static_binding; /* 1 if the tile count per feature was fixed at emit time */
   int32_t num_candidates; /* schedules compiled in; == num_features unless a tuning build */
   int32_t xcd_segments;   /* default of recom_process_args.xcd_segments (0 = flat tile walk) */
@@ -116,7 +117,9 @@ typedef struct recom_process_args {
    * (RecFlex/code_emitter/codegen.py:416-421). */
   float *d_output;
   int32_t batch;
-  /* memory traffic per tile for the run-time binding; 0 = the emitted default */
+  /* memory traffic per tile for the run-time binding; 0 = the emitted default
+   * (recom_info.tile_bytes; if that is 0 too, the device sizes the tiles from the batch:
+   * total traffic / (64 tiles per workgroup of the grid), within 64..256 KiB) */
   int32_t tile_bytes;
   /* persistent grid size; 0 = recom_get_max_concurrent_blocks() */
   int32_t grid_blocks;

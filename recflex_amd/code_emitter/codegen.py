@@ -155,7 +155,7 @@ constexpr int {vars_.EMBED_DIM_SUM} = {embed_dim_offsets[-1]};
 constexpr int {vars_.BLOCK_THREADS} = {self.block_threads};
 constexpr int {vars_.out_vec} = {self.out_vec()};
 constexpr int OCCUPANCY = {occupancy if occupancy else 0};
-constexpr int TILE_BYTES = {tile_bytes if tile_bytes else DEFAULT_TILE_BYTES};
+constexpr int TILE_BYTES = {tile_bytes if tile_bytes else 0};     // 0: chosen per batch (rfx::kAutoTile*)
 constexpr int NUM_BODIES = {len(body_ids)};
 constexpr int NUM_CANDIDATES = {len(flat)};
 constexpr int XCDS = {XCD_COUNT};

@@ -423,6 +423,21 @@ class KernelTimer:
 
 
 MAX_TILE_FACTOR = 8      # rfx::kMaxTileFactor
+AUTO_TILES_PER_WORKGROUP = 64                       # rfx::kAutoTilesPerWorkgroup
+AUTO_TILE_MIN, AUTO_TILE_MAX = 64 * 1024, 256 * 1024    # rfx::kAutoTileMin / kAutoTileMax
+
+
+def auto_tile_bytes(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int],
+                    bag_bytes: Sequence[int], grid_blocks: int) -> int:
+    """Host restatement of the tile size the device picks when none is given: the batch's
+    traffic over 64 tiles per workgroup of the grid, within 64..256 KiB, in steps of 4 KiB."""
+    total = 0
+    for off, lb, bb in zip(offsets, lookup_bytes, bag_bytes):
+        batch = len(off) - 1
+        if batch > 0:
+            total += int(off[-1] - off[0]) * lb + batch * bb
+    t = total // (max(1, grid_blocks) * AUTO_TILES_PER_WORKGROUP)
+    return min(max(t, AUTO_TILE_MIN), AUTO_TILE_MAX) & ~4095
 
 
 def tiles_per_feature(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int],

@@ -289,3 +289,20 @@ def test_profiler_command_uses_absolute_paths(tmp_path, monkeypatch):
         value = args[args.index(flag) + 1]
         assert os.path.isabs(value) and value.startswith(str(tmp_path))
     assert os.path.isabs(args[1]) and args[1].endswith("run_script.py")
+
+
+def test_automatic_tile_size_rule():
+    """The tile size the device chooses when none is given, restated on the host: 64 tiles per
+    workgroup of the grid, clamped to 64..256 KiB, multiples of 4 KiB."""
+    from recflex_amd.tuning.measure import auto_tile_bytes
+    off = lambda n_bags, per_bag: np.arange(n_bags + 1, dtype=np.int64) * per_bag
+    # tiny batch: the lower bound
+    assert auto_tile_bytes([off(512, 4)] * 4, [132] * 4, [132] * 4, 1024) == 64 * 1024
+    # 10.5 GB over 1280 workgroups: 128 KiB after rounding down to 4 KiB
+    got = auto_tile_bytes([off(16384, 20)] * 200, [148] * 200, [516] * 200, 1280)
+    total = 200 * (16384 * 20 * 148 + 16384 * 516)
+    assert got == (total // (1280 * 64)) & ~4095 and 64 * 1024 < got < 256 * 1024 and got % 4096 == 0
+    # tens of GB: the upper bound
+    assert auto_tile_bytes([off(8192, 300)] * 400, [516] * 400, [516] * 400, 1024) == 256 * 1024
+    # a grid of one workgroup and an empty batch do not divide by zero
+    assert auto_tile_bytes([np.zeros(1, dtype=np.int64)], [36], [36], 0) == 64 * 1024
