@@ -85,6 +85,8 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
 // production build, the whole candidate list in a tuning build); choice[f] (clamped; 0 if
 // choice is null) selects the one this launch runs, and cand_gran[] gives the bags a workgroup
 // of that schedule handles per pass (tiles are whole multiples of it unless a pass is too large).
+// tile_bytes: traffic a tile should carry; <= 0 lets the workgroup size the tiles from the batch
+// (see kAutoTilesPerWorkgroup above).
 // fixed_tiles: if non-null, the tile count per feature is taken from it instead of from the
 // live offsets (static thread binding, for the ablation).
 // Returns the total number of tiles.  Ends with a barrier.
