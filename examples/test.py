@@ -32,6 +32,7 @@ from recflex_amd.parser import parse_raw_data_batches, parse_table_shapes
 from recflex_amd.utils import import_from_path, find_file, compile_build
 from recflex_amd.hip_helper import HipProfiler
 from recflex_amd.schedules import default_schedule
+from recflex_amd.model_build import DEFAULT_XCD_SEGMENTS
 
 from tune import create_tuner
 
@@ -57,7 +58,8 @@ def build_targets(args: argparse.Namespace, tuner) -> str:
         mean_lens = [float(np.mean([len(i) / max(1, len(o) - 1) for i, o in feat])) for feat in tuner.batches]
         feat_schedules = [default_schedule(meta, pf, tuner.basic.block_threads)
                           for meta, pf in zip(tuner.metas, mean_lens)]
-        tuner.emit_codes(args.output_dir, feat_schedules, args.occupancy, debug=args.debug)
+        tuner.emit_codes(args.output_dir, feat_schedules, args.occupancy, debug=args.debug,
+                         xcd_segments=DEFAULT_XCD_SEGMENTS)
         compile_build(build_dir)
     return build_dir
 

@@ -8,7 +8,7 @@ its library is missing.  Names:
 ``cN_tuned``       CN with the schedules, occupancy and launch parameters recorded in
                    ``recflex_amd/tuned/cN_schedule.json`` (written by ``examples/tune.py``); the
                    default build if that file is absent
-``c3_xcd``         C3 with the XCD-aware tile walk switched on (for comparison)
+``c3_flat``        C3 with the flat tile walk instead of the XCD-segmented one (for comparison)
 ``c2s`` .. ``c5s``   shrunken C2..C5 (fewer rows / features / samples) that a CPU checker can follow
 ``variants``       one feature per (element type, dim, schedule candidate) over a spread of the
                    candidate space of all four templates, with ragged bags (up to ~1500 lookups)
@@ -78,6 +78,8 @@ def _tuned(wl: Workload, fname: str) -> ModelSpec:
         kwargs["tile_bytes"] = doc["tile_bytes"]
     if isinstance(doc, dict) and doc.get("xcd_segments", 0) > 0:
         kwargs.update(xcd_aware=True, xcd_segments=doc["xcd_segments"])
+    else:
+        kwargs.update(xcd_aware=False)      # the tuned walk is the flat one
     return ModelSpec(wl, fs, occupancy, kwargs)
 
 
@@ -142,7 +144,7 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c3_tuned": lambda: _tuned(make_workload("C3"), "c3_schedule.json"),
     "c4_tuned": lambda: _tuned(make_workload("C4"), "c4_schedule.json"),
     "c5_tuned": lambda: _tuned(make_workload("C5"), "c5_schedule.json"),
-    "c3_xcd": lambda: _default(make_workload("C3"), xcd_aware=True),
+    "c3_flat": lambda: _default(make_workload("C3"), xcd_aware=False),
     "c2s": lambda: _default(make_workload("C2", batch=512, max_rows=200_000)),
     "c3s": lambda: _default(make_workload("C3", batch=192, max_rows=60_000)),
     "c4s": lambda: _default(make_workload("C4", batch=128, num_features=48, max_rows=30_000)),
