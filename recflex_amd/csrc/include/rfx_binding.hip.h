@@ -99,72 +99,73 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
   static_assert(BT <= 16 * 64, "partial sums: at most 16 wavefronts");
   const int tid = threadIdx.x;
   const int B = io.batch;
-  int tile_size = tile_bytes;
-  const bool counted = tile_bytes <= 0 && !fixed_tiles;
-  if (counted) {
-    // first pass over the features: their live lookup counts (kept in LDS for the second pass)
-    // and the traffic of the whole batch
-    long long mine = 0;
+
+  // tiles of every feature this thread is responsible for (tid, tid + BT, ...) at the given
+  // tile size; returns the traffic of those features
+  auto bind_features = [&](const int tile_size) {
+    long long traffic = 0;
     for (int f = tid; f < F; f += BT) {
-      const int *offs = io.offsets(f);
-      const int lookups = offs[B] - offs[0];
-      s.bags_per_tile[f] = lookups;
-      mine += static_cast<long long>(lookups) * lookup_bytes[f] +
-              static_cast<long long>(B) * bag_bytes[f];
+      const int first = cand_begin[f];
+      const int ncand = cand_begin[f + 1] - first;
+      int pick = choice ? choice[f] : 0;
+      pick = pick < 0 ? 0 : (pick >= ncand ? ncand - 1 : pick);
+      s.cand[f] = first + pick;
+      const int g = cand_gran[first + pick];
+      int64_t want;
+      int64_t bag_cost = 0;       // mean traffic of one bag of this feature
+      if (fixed_tiles) {
+        want = fixed_tiles[f];
+      } else {
+        const int *offs = io.offsets(f);
+        const int64_t lookups = static_cast<int64_t>(offs[B]) - offs[0];
+        const int64_t cost = lookups * lookup_bytes[f] + static_cast<int64_t>(B) * bag_bytes[f];
+        traffic += cost;
+        want = (cost + tile_size - 1) / tile_size;
+        bag_cost = B > 0 ? cost / B : 0;
+      }
+      int tiles = want < 1 ? 1 : (want > B ? B : static_cast<int>(want));
+      int bpt = 0;
+      if (B > 0) {
+        bpt = (B + tiles - 1) / tiles;
+        // Tiles are whole workgroup passes (g bags) -- unless one pass of this schedule is more
+        // than kMaxTileFactor times the traffic a tile should carry: then the tile keeps its
+        // share of the traffic and some of the schedule's teams idle.
+        const int whole = (bpt + g - 1) / g * g;
+        if (fixed_tiles || bpt >= g ||
+            static_cast<int64_t>(whole) * bag_cost <= static_cast<int64_t>(kMaxTileFactor) * tile_size)
+          bpt = whole;
+        tiles = (B + bpt - 1) / bpt;
+      } else {
+        tiles = 0;
+      }
+      s.bags_per_tile[f] = bpt;
+      s.prefix[f + 1] = tiles;
     }
+    return traffic;
+  };
+
+  // Automatic tile size: bind with the smallest size and add up the batch's traffic on the
+  // way; only a batch large enough for bigger tiles is bound a second time.
+  const bool automatic = tile_bytes <= 0 && !fixed_tiles;
+  long long traffic = bind_features(automatic ? kAutoTileMin : tile_bytes);
+  if (automatic) {
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) mine += __shfl_xor(mine, d, 64);
-    if ((tid & 63) == 0) s.partial[tid >> 6] = mine;
-    __syncthreads();
+    for (int d = 32; d >= 1; d >>= 1) traffic += __shfl_xor(traffic, d, 64);
+    if ((tid & 63) == 0) s.partial[tid >> 6] = traffic;
+  }
+  if (tid == 0) s.prefix[0] = 0;
+  __syncthreads();
+  if (automatic) {
     long long total = 0;
     for (int w = 0; w < BT / 64; ++w) total += s.partial[w];
     long long t = total / (static_cast<long long>(gridDim.x) * kAutoTilesPerWorkgroup);
     t = t < kAutoTileMin ? kAutoTileMin : (t > kAutoTileMax ? kAutoTileMax : t);
-    tile_size = static_cast<int>(t) & ~4095;
-  }
-  for (int f = tid; f < F; f += BT) {
-    const int first = cand_begin[f];
-    const int ncand = cand_begin[f + 1] - first;
-    int pick = choice ? choice[f] : 0;
-    pick = pick < 0 ? 0 : (pick >= ncand ? ncand - 1 : pick);
-    s.cand[f] = first + pick;
-    const int g = cand_gran[first + pick];
-    int64_t want;
-    int64_t bag_cost = 0;       // mean traffic of one bag of this feature
-    if (fixed_tiles) {
-      want = fixed_tiles[f];
-    } else {
-      int64_t lookups;
-      if (counted) {
-        lookups = s.bags_per_tile[f];        // this thread's own entry of the first pass
-      } else {
-        const int *offs = io.offsets(f);
-        lookups = static_cast<int64_t>(offs[B]) - offs[0];
-      }
-      const int64_t cost = lookups * lookup_bytes[f] + static_cast<int64_t>(B) * bag_bytes[f];
-      want = (cost + tile_size - 1) / tile_size;
-      bag_cost = B > 0 ? cost / B : 0;
+    const int tile_size = static_cast<int>(t) & ~4095;
+    if (tile_size != kAutoTileMin) {      // the same decision in every thread of the grid
+      bind_features(tile_size);
+      __syncthreads();
     }
-    int tiles = want < 1 ? 1 : (want > B ? B : static_cast<int>(want));
-    int bpt = 0;
-    if (B > 0) {
-      bpt = (B + tiles - 1) / tiles;
-      // Tiles are whole workgroup passes (g bags) -- unless one pass of this schedule is more
-      // than kMaxTileFactor times the traffic a tile should carry: then the tile keeps its
-      // share of the traffic and some of the schedule's teams idle.
-      const int whole = (bpt + g - 1) / g * g;
-      if (fixed_tiles || bpt >= g ||
-          static_cast<int64_t>(whole) * bag_cost <= static_cast<int64_t>(kMaxTileFactor) * tile_size)
-        bpt = whole;
-      tiles = (B + bpt - 1) / bpt;
-    } else {
-      tiles = 0;
-    }
-    s.bags_per_tile[f] = bpt;
-    s.prefix[f + 1] = tiles;
   }
-  if (tid == 0) s.prefix[0] = 0;
-  __syncthreads();
   if (tid < 64) {
     int carry = 0;
     for (int c = 0; c < F; c += 64) {
