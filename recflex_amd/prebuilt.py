@@ -14,6 +14,7 @@ its library is missing.  Names:
                    candidate space of all four templates, with ragged bags (up to ~1500 lookups)
                    and integer-valued tables, so that sums are exact in any order
 ``edge``           dims that force 8- and 4-byte row vectors and unaligned output columns
+``wide``           1 500 small features (several binding rounds per thread)
 """
 
 import json
@@ -134,6 +135,20 @@ def _other_block_size(block_threads: int) -> ModelSpec:
     return ModelSpec(wl, fs, None)
 
 
+def _wide() -> ModelSpec:
+    """1 500 small features: several rounds of the binding loop per thread and a prefix array
+    longer than a wavefront scan covers at once, as in the reference's own models."""
+    rng = np.random.default_rng(1500)
+    feats = []
+    for i in range(1500):
+        dim = int(rng.choice([4, 8, 16, 32, 64]))
+        mean = float(rng.choice([1.0, 1.0, 3.0, 12.0, 40.0]))
+        feats.append(FeatureSpec(int(rng.integers(64, 512)), dim, "float", mean, mean == 1.0,
+                                 0.0 if mean == 1.0 else 0.3, 1.05))
+    wl = Workload("wide", 40, 1500, tuple(feats), "integer")
+    return _default(wl)
+
+
 _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c1": lambda: _default(make_workload("C1")),
     "c2": lambda: _default(make_workload("C2")),
@@ -151,6 +166,7 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c5s": lambda: _default(make_workload("C5", batch=256, num_features=24, max_rows=50_000)),
     "variants": _variants,
     "edge": _edge,
+    "wide": _wide,
     "b128": lambda: _other_block_size(128),
     "b512": lambda: _other_block_size(512),
 }
