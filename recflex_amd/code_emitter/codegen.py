@@ -37,6 +37,9 @@ INDEX_BYTES = 4
 # trip), expressed here as extra bytes so that tiles of narrow-row features do not run longer
 # than tiles of wide-row features.
 LOOKUP_OVERHEAD_BYTES = 0
+# models of more features than this are bound once per launch by a small kernel instead of by
+# every workgroup of the fused kernel (rfx::bind_once)
+BIND_ONCE_MIN_FEATS = 2048
 
 
 def _c_array(ctype: str, name: str, values: List[int], per_line: int = 16) -> str:
@@ -149,6 +152,8 @@ class CodeEmitter:
         id_map, body_ids = self.dedup()
         flat, cand_begin = self.flat_candidates()
         embed_dim_offsets = self.embed_dim_offsets()
+        bind_once = num_feats > BIND_ONCE_MIN_FEATS
+        fixed_arg = "c_fixed_task_block_nums" if fixed_task_block_nums else "nullptr"
 
         consts = f'''constexpr int NUM_FEATS = {num_feats};
 constexpr int {vars_.EMBED_DIM_SUM} = {embed_dim_offsets[-1]};
@@ -162,6 +167,8 @@ constexpr int XCDS = {XCD_COUNT};
 constexpr int XCD_SEGMENTS = {xcd_segments if xcd_aware else 0};
 constexpr bool TIMING = {"true" if timing else "false"};
 constexpr bool STATIC_BINDING = {"true" if fixed_task_block_nums else "false"};
+#define RFX_BIND_ONCE {1 if bind_once else 0}
+constexpr bool BIND_ONCE = RFX_BIND_ONCE;
 
 '''
 
@@ -240,7 +247,39 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
 
         launch_bounds = (f"__launch_bounds__({vars_.BLOCK_THREADS}, {occupancy})" if occupancy
                          else f"__launch_bounds__({vars_.BLOCK_THREADS})")
-        kernel = f'''
+        if bind_once:
+            bind_decl = "  __shared__ rfx::PrefixStorage<NUM_FEATS> s_bind;\n"
+            bind_call = (f"  const int total_tiles = rfx::load_prefix<NUM_FEATS, {vars_.BLOCK_THREADS}>"
+                         "(s_bind, d_bound);\n  (void)tile_bytes;\n  (void)d_schedule_choice;")
+            bound_src = "d_bound->"
+        else:
+            bind_decl = "  __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;\n"
+            bind_call = (f"  const int total_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}>(\n"
+                         "      s_bind, io, tile_bytes, c_lookup_bytes, c_bag_bytes, c_cand_begin, c_cand_gran,\n"
+                         f"      d_schedule_choice, {fixed_arg}, gridDim.x);\n  (void)d_bound;")
+            bound_src = "s_bind."
+        bind_kernel = f'''
+// the binding tables of the launches in flight, one slot per stream (rfx::bind_slot_for)
+static __device__ __align__(256) char
+    g_bound[BIND_ONCE ? rfx::kBindSlots * sizeof(rfx::BoundTables<NUM_FEATS>) : 256];
+
+// One workgroup binds the whole model for this launch (models of thousands of features).
+extern "C" __global__ void __launch_bounds__(1024) BindKnl(
+    const int64_t *__restrict__ d_io_ptrs, const char *__restrict__ d_arg_buffers,
+    const int64_t *__restrict__ d_arg_buffer_offsets, const int batch, const int tile_bytes,
+    const int *__restrict__ d_schedule_choice, const int grid_blocks,
+    rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound) {{
+  __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;
+  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
+  rfx::bind_once<NUM_FEATS, 1024>(s_bind, d_bound, io, tile_bytes, c_lookup_bytes, c_bag_bytes,
+                                  c_cand_begin, c_cand_gran, d_schedule_choice, {fixed_arg},
+                                  grid_blocks);
+}}
+''' if bind_once else '''
+static __device__ __align__(256) char g_bound[256];     // unused: every workgroup binds for itself
+'''
+
+        kernel = bind_kernel + f'''
 extern "C" __global__ void {launch_bounds} FusedKnl(
     const int64_t *__restrict__ d_embed_table_ptrs,
     const int64_t *__restrict__ d_io_ptrs,
@@ -249,15 +288,13 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     float *__restrict__ d_output,
     const int batch, const int tile_bytes, const int xcd_segments,
     const int *__restrict__ d_schedule_choice,
-    unsigned long long *__restrict__ d_times, const int {vars_.out_row_stride}) {{
-  __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;
-
+    unsigned long long *__restrict__ d_times, const int {vars_.out_row_stride},
+    const rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound) {{
+{bind_decl}
   __shared__ KnlTempStorage s;
 {stage_decl}{timing_init}
   const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
-  const int total_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}>(
-      s_bind, io, tile_bytes, c_lookup_bytes, c_bag_bytes, c_cand_begin, c_cand_gran,
-      d_schedule_choice, {"c_fixed_task_block_nums" if fixed_task_block_nums else "nullptr"});
+{bind_call}
 
   // Tiles are ordered by feature.  Workgroup i runs on XCD i % XCDS.  With xcd_segments > 0 the
   // tile space is cut into XCDS * xcd_segments equal segments and segment s belongs to XCD
@@ -282,8 +319,8 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
       if (tile >= total_tiles) continue;
     }}
 {timing_begin if timing and timing_branch else ''}
-    const int feat_idx = __builtin_amdgcn_readfirstlane(rfx::find_feature<NUM_FEATS>(s_bind, tile));
-    const int bags_per_tile = s_bind.bags_per_tile[feat_idx];
+    const int feat_idx = __builtin_amdgcn_readfirstlane(rfx::find_feature<NUM_FEATS>(s_bind.prefix, tile));
+    const int bags_per_tile = {bound_src}bags_per_tile[feat_idx];
     const int {vars_.bag_begin} = (tile - s_bind.prefix[feat_idx]) * bags_per_tile;
     const int {vars_.bag_end} = min(batch, {vars_.bag_begin} + bags_per_tile);
     const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[feat_idx]);
@@ -291,7 +328,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     const int *offsets = io.offsets(feat_idx);
     const int embed_dim_offset = c_embed_dim_offsets[feat_idx];
 {timing_begin if timing and not timing_branch else ''}
-    switch (c_cand_func_ids[s_bind.cand[feat_idx]]) {{
+    switch (c_cand_func_ids[{bound_src}cand[feat_idx]]) {{
 {cases}      default: break;
     }}
 {timing_end}
@@ -331,12 +368,29 @@ extern "C" int recom_process(const recom_process_args *a) {
   const char *arg_buffers = static_cast<const char *>(a->d_arg_buffers);
   int batch = a->batch, tile_arg = tile_bytes, xcd_arg = xcd_segments;
   int stride_arg = static_cast<int>(row_stride);
+  void *bound = nullptr;
+#if RFX_BIND_ONCE
+  e = rfx::bind_slot_for(
+      [](char **p) {
+        return hipGetSymbolAddress(reinterpret_cast<void **>(p), HIP_SYMBOL(g_bound));
+      },
+      sizeof(rfx::BoundTables<NUM_FEATS>), a->stream, &bound);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (!bound) return static_cast<int>(hipErrorOutOfMemory);    // more streams than slots
+  int grid_arg = grid;
+  void *bind_args[] = {const_cast<int64_t **>(&a->d_io_ptrs), &arg_buffers,
+                       const_cast<int64_t **>(&a->d_arg_buffer_offsets), &batch, &tile_arg,
+                       const_cast<int32_t **>(&a->d_schedule_choice), &grid_arg, &bound};
+  e = hipLaunchKernel(reinterpret_cast<const void *>(BindKnl), dim3(1), dim3(1024), bind_args, 0,
+                      static_cast<hipStream_t>(a->stream));
+  if (e != hipSuccess) return static_cast<int>(e);
+#endif
   void *kernel_args[] = {
       const_cast<int64_t **>(&a->d_embed_table_ptrs), const_cast<int64_t **>(&a->d_io_ptrs),
       &arg_buffers, const_cast<int64_t **>(&a->d_arg_buffer_offsets),
       const_cast<float **>(&a->d_output), &batch, &tile_arg, &xcd_arg,
       const_cast<int32_t **>(&a->d_schedule_choice),
-      const_cast<unsigned long long **>(&a->d_times), &stride_arg};
+      const_cast<unsigned long long **>(&a->d_times), &stride_arg, &bound};
   e = hipLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
                       kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream));
   return static_cast<int>(e);

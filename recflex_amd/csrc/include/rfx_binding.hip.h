@@ -89,13 +89,15 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
 // (see kAutoTilesPerWorkgroup above).
 // fixed_tiles: if non-null, the tile count per feature is taken from it instead of from the
 // live offsets (static thread binding, for the ablation).
+// grid_blocks: workgroups of the fused kernel's grid (for the automatic tile size).
 // Returns the total number of tiles.  Ends with a barrier.
 template <int F, int BT>
 __device__ __forceinline__ int
 bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
            const int *__restrict__ lookup_bytes, const int *__restrict__ bag_bytes,
            const int *__restrict__ cand_begin, const int *__restrict__ cand_gran,
-           const int *__restrict__ choice, const int *__restrict__ fixed_tiles) {
+           const int *__restrict__ choice, const int *__restrict__ fixed_tiles,
+           const int grid_blocks) {
   static_assert(BT <= 16 * 64, "partial sums: at most 16 wavefronts");
   const int tid = threadIdx.x;
   const int B = io.batch;
@@ -158,7 +160,7 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
   if (automatic) {
     long long total = 0;
     for (int w = 0; w < BT / 64; ++w) total += s.partial[w];
-    long long t = total / (static_cast<long long>(gridDim.x) * kAutoTilesPerWorkgroup);
+    long long t = total / (static_cast<long long>(grid_blocks) * kAutoTilesPerWorkgroup);
     t = t < kAutoTileMin ? kAutoTileMin : (t > kAutoTileMax ? kAutoTileMax : t);
     const int tile_size = static_cast<int>(t) & ~4095;
     if (tile_size != kAutoTileMin) {      // the same decision in every thread of the grid
@@ -182,13 +184,61 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
 
 // feature owning global tile id `tile` (0 <= tile < prefix[F]): largest f with prefix[f] <= tile
 template <int F>
-__device__ __forceinline__ int find_feature(const BindingStorage<F> &s, const int tile) {
+__device__ __forceinline__ int find_feature(const int *prefix, const int tile) {
   int lo = 0, hi = F;
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
-    if (s.prefix[mid] <= tile) lo = mid; else hi = mid;
+    if (prefix[mid] <= tile) lo = mid; else hi = mid;
   }
   return lo;
+}
+template <int F>
+__device__ __forceinline__ int find_feature(const BindingStorage<F> &s, const int tile) {
+  return find_feature<F>(s.prefix, tile);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Binding computed once per launch, for models of thousands of features.  The binding costs
+// every workgroup some 10 us per thousand features and 12 bytes of LDS per feature; at 10 000
+// features that is 100 us per workgroup and 120 KB, which leaves one workgroup per CU.  Such a
+// model is bound by one workgroup of a small kernel launched ahead of the fused one
+// (bind_once), into a table in device memory; the workgroups of the fused kernel copy only the
+// prefix array into LDS (load_prefix) and read the two other entries of a tile's feature from
+// the table.
+// ---------------------------------------------------------------------------------------------
+template <int F> struct BoundTables {       // in device memory
+  int prefix[F + 1];
+  int bags_per_tile[F];
+  int cand[F];
+};
+
+template <int F> struct PrefixStorage {     // what a workgroup of the fused kernel keeps in LDS
+  int prefix[F + 1];
+};
+
+template <int F, int BT>
+__device__ __forceinline__ void
+bind_once(BindingStorage<F> &s, BoundTables<F> *__restrict__ out, const IoView &io,
+          const int tile_bytes, const int *__restrict__ lookup_bytes,
+          const int *__restrict__ bag_bytes, const int *__restrict__ cand_begin,
+          const int *__restrict__ cand_gran, const int *__restrict__ choice,
+          const int *__restrict__ fixed_tiles, const int grid_blocks) {
+  bind_tiles<F, BT>(s, io, tile_bytes, lookup_bytes, bag_bytes, cand_begin, cand_gran, choice,
+                    fixed_tiles, grid_blocks);
+  for (int f = threadIdx.x; f < F; f += BT) {
+    out->bags_per_tile[f] = s.bags_per_tile[f];
+    out->cand[f] = s.cand[f];
+  }
+  for (int f = threadIdx.x; f <= F; f += BT) out->prefix[f] = s.prefix[f];
+}
+
+// Returns the total number of tiles.  Ends with a barrier.
+template <int F, int BT>
+__device__ __forceinline__ int load_prefix(PrefixStorage<F> &s,
+                                           const BoundTables<F> *__restrict__ bound) {
+  for (int f = threadIdx.x; f <= F; f += BT) s.prefix[f] = bound->prefix[f];
+  __syncthreads();
+  return s.prefix[F];
 }
 
 } // namespace rfx

@@ -15,6 +15,7 @@ its library is missing.  Names:
                    and integer-valued tables, so that sums are exact in any order
 ``edge``           dims that force 8- and 4-byte row vectors and unaligned output columns
 ``wide``           1 500 small features (several binding rounds per thread)
+``wider``          2 500 small features (bound once per launch by the binding kernel)
 """
 
 import json
@@ -135,17 +136,19 @@ def _other_block_size(block_threads: int) -> ModelSpec:
     return ModelSpec(wl, fs, None)
 
 
-def _wide() -> ModelSpec:
-    """1 500 small features: several rounds of the binding loop per thread and a prefix array
-    longer than a wavefront scan covers at once, as in the reference's own models."""
-    rng = np.random.default_rng(1500)
+def _wide(num_features: int = 1500, name: str = "wide") -> ModelSpec:
+    """Many small features: several rounds of the binding loop per thread and a prefix array
+    longer than a wavefront scan covers at once, as in the reference's own models.  Above
+    ``codegen.BIND_ONCE_MIN_FEATS`` features the binding is computed once per launch by a kernel
+    of its own (``wider``)."""
+    rng = np.random.default_rng(num_features)
     feats = []
-    for i in range(1500):
+    for i in range(num_features):
         dim = int(rng.choice([4, 8, 16, 32, 64]))
         mean = float(rng.choice([1.0, 1.0, 3.0, 12.0, 40.0]))
         feats.append(FeatureSpec(int(rng.integers(64, 512)), dim, "float", mean, mean == 1.0,
                                  0.0 if mean == 1.0 else 0.3, 1.05))
-    wl = Workload("wide", 40, 1500, tuple(feats), "integer")
+    wl = Workload(name, 40, num_features, tuple(feats), "integer")
     return _default(wl)
 
 
@@ -167,6 +170,7 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "variants": _variants,
     "edge": _edge,
     "wide": _wide,
+    "wider": lambda: _wide(2500, "wider"),
     "b128": lambda: _other_block_size(128),
     "b512": lambda: _other_block_size(512),
 }
