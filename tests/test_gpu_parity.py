@@ -204,10 +204,12 @@ def test_every_schedule_variant_on_ragged_batches(batch, seed):
     assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
 
 
-def test_launch_replays_inside_a_hip_graph():
+@pytest.mark.parametrize("name", ["c3s", "wider"])
+def test_launch_replays_inside_a_hip_graph(name):
     """recom_process is a single kernel launch on the caller's stream (binding happens on the
     device, no host-side task mapping, no copies), so a serving loop can capture it once and
-    replay it.  Captured after one eager call; replayed four times, each time with new bag
+    replay it (a library of more than 2 048 features launches its binding kernel first: two
+    kernel nodes).  Captured after one eager call; replayed four times, each time with new bag
     lengths and lookups written into the same index / offset buffers, with eager work and
     synchronisations in between; every replay is compared bit for bit with an eager launch."""
     import torch
@@ -215,9 +217,9 @@ def test_launch_replays_inside_a_hip_graph():
     from recflex_amd.rec_modules import FeatEmbed
     from recflex_amd.workloads import gen_inputs, gen_tables
 
-    wl = prebuilt.model_spec("c3s").workload
+    wl = prebuilt.model_spec(name).workload
     dev = torch.device("cuda", 0)
-    print(f"[case] c3s captured in a graph: F={wl.num_features} B={wl.batch}", flush=True)
+    print(f"[case] {name} captured in a graph: F={wl.num_features} B={wl.batch}", flush=True)
     tables = gen_tables(wl, dev)
     batches = [gen_inputs(wl._replace(seed=wl.seed + 31 * k)) for k in range(4)]
     capacity = [max(len(b[0][f]) for b in batches) for f in range(wl.num_features)]
@@ -232,7 +234,7 @@ def test_launch_replays_inside_a_hip_graph():
             d_idx[f][:len(indices[f])].copy_(torch.from_numpy(indices[f]))
             d_off[f].copy_(torch.from_numpy(offsets[f]))
 
-    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib("c3s"))
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib(name))
     load(batches[0])
     layer.forward_indices(d_idx, d_off, out=eager_out)       # first call: launch state, addresses
     torch.cuda.synchronize()
