@@ -149,7 +149,11 @@ typedef struct recom_process_args {
 /* Launch the fused kernel: for every feature f and sample b,
  *   output[b, off_f : off_f + D_f] = sum_{p in [offsets_f[b], offsets_f[b+1])} row(table_f, indices_f[p])
  * Asynchronous.  Replaces torch.ops.recom.process (RecFlex/code_emitter/codegen.py:403-444)
- * and FusedKnl (RecFlex/code_emitter/codegen.py:318-383). */
+ * and FusedKnl (RecFlex/code_emitter/codegen.py:318-383).
+ * Never allocates.  A library of more than 2048 features launches a one-workgroup kernel ahead
+ * of the fused one that binds the model for this batch into a static device array of the
+ * library; the array has one slot per stream (eight), launches on one stream share theirs, and
+ * a ninth stream on the same device is refused with hipErrorOutOfMemory (2). */
 int recom_process(const recom_process_args *args);
 
 /* ------------------------------------------------------------------------------------------
