@@ -58,7 +58,7 @@ typedef struct recom_info {
   int32_t reserved[5];
 } recom_info;
 
-#define RECOM_ABI_VERSION 2
+#define RECOM_ABI_VERSION 3     /* 3: recom_get_workspace_bytes, d_workspace / workspace_bytes */
 
 /* Static description of the emitted kernel.  No reference counterpart as a function: the
  * reference bakes the same numbers into process.cu (EMBED_DIM_SUM, block_threads,
@@ -83,6 +83,12 @@ int recom_get_candidate_counts(int32_t *counts);
  * persistent grid.  Replaces torch.ops.recom.get_max_concurrent_blocks
  * (RecFlex/code_emitter/codegen.py:446-452, RecFlex/sched_basic_csrc/include/utils.cuh:6-21). */
 int recom_get_max_concurrent_blocks(int32_t *out);
+
+/* Bytes of recom_process_args.d_workspace this library needs: 0 unless a feature runs a
+ * schedule that splits bags over workgroups, then 2048 * (D_f + 1) * 4 bytes for each such
+ * feature (rounded up to 128).  Replaces the extra-buffer sizes the reference's host
+ * preprocessors report per batch (RecFlex/code_emitter/codegen.py:149-160, extra_buffer_offsets). */
+int recom_get_workspace_bytes(int64_t *out);
 
 typedef struct recom_launch_info {
   int32_t compute_units;      /* CUs of the current device */
@@ -144,6 +150,16 @@ typedef struct recom_process_args {
    * slabs into one [batch, sum of all] buffer.  Must be a multiple of 4 when embed_dim_sum is
    * (the kernel then stores 16 bytes at a time), and d_output aligned likewise. */
   int64_t output_row_stride;
+  /* Workspace of the schedules that give one bag to several workgroups (batches of few, very
+   * long bags): device memory of at least recom_get_workspace_bytes() bytes, 16-byte aligned,
+   * caller allocated.  It must be all zero before the first launch that uses it; every launch
+   * leaves its arrival counters at zero again, so it is cleared once, not per launch.  Launches
+   * that may overlap (different streams) need a workspace each.  Ignored (may be NULL) by a
+   * library whose recom_get_workspace_bytes() is 0.  The reference's counterparts are the
+   * extra_buffers / task_barriers tensors of torch.ops.recom.process
+   * (RecFlex/code_emitter/codegen.py:403-444, RecFlex/rec_modules.py:44-52). */
+  void *d_workspace;
+  int64_t workspace_bytes;
 } recom_process_args;
 
 /* Launch the fused kernel: for every feature f and sample b,

@@ -22,7 +22,7 @@ import json
 import os
 from typing import Any, Dict, List, NamedTuple, Tuple
 
-from .schedule_base import ScheduleBase, ScheduleVars, PreprocessVars
+from .schedule_base import ScheduleBase, ScheduleVars, PreprocessVars, SPLIT_MAX_TILES, SPLIT_GRANULARITY
 from .build_basic import BasicBuilder
 
 # memory traffic (bytes) the run-time binding aims at per tile
@@ -118,6 +118,18 @@ class CodeEmitter:
             begin.append(len(flat))
         return flat, begin
 
+    def split_regions(self) -> Tuple[List[int], int]:
+        """Workspace of the schedules that split bags over workgroups: the first float of each
+        feature's region (-1 for a feature none of whose candidates needs one; a feature's
+        candidates share its region, only one of them runs in a launch) and the total floats."""
+        regions, total = [], 0
+        for cands in self.feat_candidates:
+            need = max(schedule.WorkspaceFloats(params) for schedule, params in cands)
+            need = (need + 31) // 32 * 32          # regions start on 128-byte boundaries
+            regions.append(total if need else -1)
+            total += need
+        return regions, total
+
     def dedup(self) -> Tuple[Dict[int, int], List[int]]:
         """candidate index -> index of the first candidate with the same (LDS type, body); list
         of those first indices.  With one schedule per feature, candidate index == feature."""
@@ -153,6 +165,8 @@ class CodeEmitter:
         flat, cand_begin = self.flat_candidates()
         embed_dim_offsets = self.embed_dim_offsets()
         bind_once = num_feats > BIND_ONCE_MIN_FEATS
+        split_regions, workspace_floats = self.split_regions()
+        has_split = workspace_floats > 0
         fixed_arg = "c_fixed_task_block_nums" if fixed_task_block_nums else "nullptr"
 
         consts = f'''constexpr int NUM_FEATS = {num_feats};
@@ -169,6 +183,11 @@ constexpr bool TIMING = {"true" if timing else "false"};
 constexpr bool STATIC_BINDING = {"true" if fixed_task_block_nums else "false"};
 #define RFX_BIND_ONCE {1 if bind_once else 0}
 constexpr bool BIND_ONCE = RFX_BIND_ONCE;
+// bytes of caller workspace the split-bag schedules need (0: no schedule splits bags)
+constexpr long long WORKSPACE_BYTES = {workspace_floats * 4}LL;
+constexpr bool HAS_SPLIT = WORKSPACE_BYTES > 0;
+static_assert(rfx::kBindMaxSplitTiles == {SPLIT_MAX_TILES} && rfx::kSplitGran == {SPLIT_GRANULARITY},
+              "workspace regions were sized for this");
 
 '''
 
@@ -186,7 +205,9 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
     float *__restrict__ {vars_.output},
     const int {vars_.out_row_stride}, const int {vars_.embed_dim_offset},
     const int {vars_.bag_begin}, const int {vars_.bag_end},
-    char *__restrict__ {vars_.shmem}, rfx::f32x4 *__restrict__ {vars_.stage}) {{
+    char *__restrict__ {vars_.shmem}, rfx::f32x4 *__restrict__ {vars_.stage},
+    const int {vars_.split_part}, const int {vars_.split_parts},
+    float *__restrict__ {vars_.split_region}) {{
   {schedule.EmitScheduleBody(params)}
 }}
 '''
@@ -201,6 +222,9 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
                             for s, _ in self.feat_schedules])
         tables += _c_array("int", "c_bag_bytes",
                            [s.meta.embed_dim * 4 + BAG_FIXED_BYTES for s, _ in self.feat_schedules])
+        if has_split:
+            # first float of each feature's region of the workspace (-1: the feature has none)
+            tables += _c_array("long long", "c_split_region", split_regions)
         if fixed_task_block_nums:
             assert len(fixed_task_block_nums) == num_feats
             tables += _c_array("int", "c_fixed_task_block_nums",
@@ -240,7 +264,8 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
         stage_decl = (f"  __shared__ rfx::TeamStage<{vars_.BLOCK_THREADS}> s_stage;\n" if need_stage else "")
         call_args = (f"table, indices, offsets, d_output, {vars_.out_row_stride}, embed_dim_offset, "
                      f"{vars_.bag_begin}, {vars_.bag_end}, reinterpret_cast<char *>(&s), "
-                     + ("&s_stage.seg[0][0]" if need_stage else "nullptr"))
+                     + ("&s_stage.seg[0][0]" if need_stage else "nullptr")
+                     + f", {vars_.split_part}, {vars_.split_parts}, {vars_.split_region}")
         cases = "".join(
             f"      case {feat_idx}: ProcessFeat{feat_idx}({call_args}); break;\n"
             for feat_idx in body_ids)
@@ -254,7 +279,7 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
             bound_src = "d_bound->"
         else:
             bind_decl = "  __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;\n"
-            bind_call = (f"  const int total_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}>(\n"
+            bind_call = (f"  const int total_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}, HAS_SPLIT>(\n"
                          "      s_bind, io, tile_bytes, c_lookup_bytes, c_bag_bytes, c_cand_begin, c_cand_gran,\n"
                          f"      d_schedule_choice, {fixed_arg}, gridDim.x);\n  (void)d_bound;")
             bound_src = "s_bind."
@@ -271,7 +296,7 @@ extern "C" __global__ void __launch_bounds__(1024) BindKnl(
     rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound) {{
   __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;
   const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
-  rfx::bind_once<NUM_FEATS, 1024>(s_bind, d_bound, io, tile_bytes, c_lookup_bytes, c_bag_bytes,
+  rfx::bind_once<NUM_FEATS, 1024, HAS_SPLIT>(s_bind, d_bound, io, tile_bytes, c_lookup_bytes, c_bag_bytes,
                                   c_cand_begin, c_cand_gran, d_schedule_choice, {fixed_arg},
                                   grid_blocks);
 }}
@@ -289,7 +314,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     const int batch, const int tile_bytes, const int xcd_segments,
     const int *__restrict__ d_schedule_choice,
     unsigned long long *__restrict__ d_times, const int {vars_.out_row_stride},
-    const rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound) {{
+    const rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound, float *__restrict__ d_workspace) {{
 {bind_decl}
   __shared__ KnlTempStorage s;
 {stage_decl}{timing_init}
@@ -321,8 +346,22 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
 {timing_begin if timing and timing_branch else ''}
     const int feat_idx = __builtin_amdgcn_readfirstlane(rfx::find_feature<NUM_FEATS>(s_bind.prefix, tile));
     const int bags_per_tile = {bound_src}bags_per_tile[feat_idx];
-    const int {vars_.bag_begin} = (tile - s_bind.prefix[feat_idx]) * bags_per_tile;
-    const int {vars_.bag_end} = min(batch, {vars_.bag_begin} + bags_per_tile);
+    int {vars_.bag_begin} = (tile - s_bind.prefix[feat_idx]) * bags_per_tile;
+    int {vars_.bag_end} = min(batch, {vars_.bag_begin} + bags_per_tile);
+    // a feature whose bags are split over workgroups: bags_per_tile = -parts, the feature's tile
+    // t is part t % parts of bag t / parts
+    int {vars_.split_part} = 0, {vars_.split_parts} = 1;
+    float *{vars_.split_region} = nullptr;
+    if constexpr (HAS_SPLIT) {{
+      if (bags_per_tile < 0) {{
+        const int local = tile - s_bind.prefix[feat_idx];
+        {vars_.split_parts} = -bags_per_tile;
+        {vars_.bag_begin} = local / {vars_.split_parts};
+        {vars_.split_part} = local - {vars_.bag_begin} * {vars_.split_parts};
+        {vars_.bag_end} = {vars_.bag_begin} + 1;
+      }}
+      {vars_.split_region} = d_workspace + {"c_split_region[feat_idx]" if has_split else "0"};
+    }}
     const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[feat_idx]);
     const int *indices = io.indices(feat_idx);
     const int *offsets = io.offsets(feat_idx);
@@ -352,6 +391,10 @@ extern "C" int recom_process(const recom_process_args *a) {
   if (row_stride < EMBED_DIM_SUM || row_stride > 0x7fffffff || row_stride % OUT_VEC != 0 ||
       reinterpret_cast<uintptr_t>(a->d_output) % (OUT_VEC * sizeof(float)) != 0)
     return static_cast<int>(hipErrorInvalidValue);
+  // split-bag schedules keep partial sums and arrival counters in the caller's workspace
+  if (HAS_SPLIT && (!a->d_workspace || a->workspace_bytes < WORKSPACE_BYTES ||
+                    reinterpret_cast<uintptr_t>(a->d_workspace) % 16 != 0))
+    return static_cast<int>(hipErrorInvalidValue);
   if (a->batch == 0) return static_cast<int>(hipSuccess);
 
   const rfx::LaunchState *st = nullptr;
@@ -368,6 +411,7 @@ extern "C" int recom_process(const recom_process_args *a) {
   const char *arg_buffers = static_cast<const char *>(a->d_arg_buffers);
   int batch = a->batch, tile_arg = tile_bytes, xcd_arg = xcd_segments;
   int stride_arg = static_cast<int>(row_stride);
+  void *workspace = a->d_workspace;
   void *bound = nullptr;
 #if RFX_BIND_ONCE
   e = rfx::bind_slot_for(
@@ -390,7 +434,7 @@ extern "C" int recom_process(const recom_process_args *a) {
       &arg_buffers, const_cast<int64_t **>(&a->d_arg_buffer_offsets),
       const_cast<float **>(&a->d_output), &batch, &tile_arg, &xcd_arg,
       const_cast<int32_t **>(&a->d_schedule_choice),
-      const_cast<unsigned long long **>(&a->d_times), &stride_arg, &bound};
+      const_cast<unsigned long long **>(&a->d_times), &stride_arg, &bound, &workspace};
   e = hipLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
                       kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream));
   return static_cast<int>(e);
@@ -413,6 +457,12 @@ extern "C" int recom_get_launch_info(recom_launch_info *out) {
   out->num_vgprs = st->num_vgprs;
   out->static_lds_bytes = st->static_lds;
   out->lds_bytes_per_cu = st->lds_per_cu;
+  return static_cast<int>(hipSuccess);
+}
+
+extern "C" int recom_get_workspace_bytes(int64_t *out) {
+  if (!out) return static_cast<int>(hipErrorInvalidValue);
+  *out = WORKSPACE_BYTES;
   return static_cast<int>(hipSuccess);
 }
 

@@ -12,6 +12,13 @@ from abc import ABC, abstractmethod
 from typing import List, NamedTuple, Tuple
 
 
+# Schedules that split a bag over several workgroups: the granularity by which such a schedule
+# announces itself to the run-time binding (rfx::kSplitGran) and the slots of a feature's
+# workspace region (rfx::kBindMaxSplitTiles)
+SPLIT_GRANULARITY = -1
+SPLIT_MAX_TILES = 2048
+
+
 class InputStats(NamedTuple):
     # field names as in the reference (including the spelling of ``minmum``)
     mean: float
@@ -102,6 +109,12 @@ class ScheduleVars(NamedTuple):
     bag_begin: str = "bag_begin"             # this tile sums bags [bag_begin, bag_end)
     bag_end: str = "bag_end"
     out_vec: str = "OUT_VEC"                 # widest aligned output store in floats (4, 2 or 1)
+    # schedules that split a bag over workgroups: this tile is part split_part of split_parts of
+    # bag bag_begin (split_parts <= 1: a plain bag range); split_region = the feature's floats
+    # of the caller's workspace (null if no schedule of the feature splits)
+    split_part: str = "split_part"
+    split_parts: str = "split_parts"
+    split_region: str = "split_region"
 
 
 class PreprocessVars(NamedTuple):
@@ -137,6 +150,11 @@ class ScheduleBase(ABC):
     @abstractmethod
     def TileGranularity(self, params: NamedTuple) -> int:
         """Bags one workgroup of this schedule covers per pass; tiles are multiples of it."""
+
+    def WorkspaceFloats(self, params: NamedTuple) -> int:
+        """Floats of the caller's workspace this schedule needs for its feature (0 = none).  A
+        schedule that needs some must return the split granularity from ``TileGranularity``."""
+        return 0
 
     @abstractmethod
     def GenParamCandidates(self, stats: InputStats = None) -> List:

@@ -8,6 +8,9 @@
 //   T == 64         wavefront-per-bag       (team_bags)
 //   T == BT (256)   block-per-bag           (block_bags: indices staged in LDS, partial sums
 //                                            of the 4 wavefronts combined through LDS)
+//   T == parts*BT   several workgroups per bag (split_bags: block_bags on a share of the bag's
+//                                            lookups, partial sums combined through a workspace
+//                                            by the workgroup that finishes last)
 //
 // Reference counterparts: ws::SparseSegmentReduce
 // (examples/csrc/include/warp_per_sample_kernel.cuh:10-82), obms::SparseSegmentReduce
@@ -18,6 +21,7 @@
 // is a range of bags [bag_begin, bag_end) chosen at run time, and U lookups x UB bags x VPP
 // vectors are kept in flight per lane.
 #pragma once
+#include "rfx_binding.hip.h"
 #include "rfx_crosslane.hip.h"
 #include "rfx_rows.hip.h"
 
@@ -317,7 +321,109 @@ template <int BT, int DT, int D, int X, int CHUNK> struct BlockBagStorage {
   int idx[CHUNK];
   float part[BT / 64][COLS];
   float part_bias[BT / 64];
+  int last;                                     // split_bags: this workgroup finishes the bag
 };
+
+// The workgroup sums the lookups [beg, end) of one bag: afterwards s.part[w][j] holds wavefront
+// w's share of column j (and s.part_bias[w] its share of the int8 biases), and a barrier has
+// made them visible to every thread.  Starts with a barrier that orders an earlier use of
+// s.part / s.idx before this one.
+template <int BT, int DT, int D, int X, int U, int CHUNK>
+__device__ __forceinline__ void
+block_sum_range(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ table,
+                const int *__restrict__ indices, const int beg, const int end, const int tid) {
+  using R = Row<DT, D>;
+  static_assert(X >= 1 && X <= 64 && (X & (X - 1)) == 0, "column lanes");
+  static_assert(BT % 64 == 0 && CHUNK % BT == 0, "chunk must be whole workgroup loads");
+  constexpr int Y = BT / X;
+  constexpr int VPL = ceil_div(R::V, X);
+  constexpr int VB = R::VB;
+  constexpr int EPV = R::EPV;
+
+  const int y = tid / X;
+  const int x = tid - y * X;
+  const int wave = tid / 64;
+  const int lane = tid - wave * 64;
+
+  float acc[VPL][EPV];
+  float bias_acc = 0.f;
+#pragma unroll
+  for (int v = 0; v < VPL; ++v)
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) acc[v][e] = 0.f;
+
+  __syncthreads();
+  for (int c0 = beg; c0 < end; c0 += CHUNK) {
+    const int n = min(CHUNK, end - c0);
+    if (c0 != beg) __syncthreads();
+#pragma unroll
+    for (int i = 0; i < CHUNK; i += BT)
+      if (i + tid < n) s.idx[i + tid] = indices[c0 + i + tid];
+    __syncthreads();
+
+    for (int base = 0; base < n; base += U * Y) {
+      Vec<VB> buf[U][VPL];
+      f32x2 sb[U];
+      bool ok[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int p = base + u * Y + y;
+        ok[u] = p < n;
+        if (ok[u]) {
+          const char *row = table + static_cast<int64_t>(s.idx[p]) * R::STRIDE;
+#pragma unroll
+          for (int v = 0; v < VPL; ++v) {
+            const int c = x + v * X;
+            if (c < R::V) buf[u][v] = load_vec<VB>(row + c * VB);
+          }
+          if constexpr (DT == I8) sb[u] = load_scale_bias<D>(row);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (ok[u]) {
+#pragma unroll
+          for (int v = 0; v < VPL; ++v) {
+            const int c = x + v * X;
+            if (c < R::V) accumulate<DT, VB>(acc[v], buf[u][v], DT == I8 ? sb[u].x : 1.f);
+          }
+          if constexpr (DT == I8) bias_acc += sb[u].y;
+        }
+    }
+  }
+
+  // combine the lookup lanes that share a wavefront
+  if constexpr (X < 64) {
+    if constexpr (DT == I8) bias_acc = reduce_over_y<X, 64>(bias_acc);
+#pragma unroll
+    for (int v = 0; v < VPL; ++v)
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) acc[v][e] = reduce_over_y<X, 64>(acc[v][e]);
+  }
+  if (lane < X) {
+#pragma unroll
+    for (int v = 0; v < VPL; ++v)
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) s.part[wave][(x + v * X) * EPV + e] = acc[v][e];
+    if (lane == 0) s.part_bias[wave] = bias_acc;
+  }
+  __syncthreads();
+}
+
+// column j of what block_sum_range left in LDS: the wavefronts' shares in wavefront order
+template <int BT, int DT, int D, int X, int CHUNK>
+__device__ __forceinline__ float
+block_column(const BlockBagStorage<BT, DT, D, X, CHUNK> &s, const int j) {
+  constexpr int WAVES = BT / 64;
+  float t = 0.f;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) t += s.part[w][j];
+  if constexpr (DT == I8) {
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) t += s.part_bias[w];
+  }
+  return t;
+}
 
 template <int BT, int DT, int D, int X, int U, int CHUNK>
 __device__ __forceinline__ void
@@ -325,104 +431,91 @@ block_bags(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ tab
            const int *__restrict__ indices, const int *__restrict__ offsets,
            float *__restrict__ out, const int esum, const int col_off, const int bag_begin,
            const int bag_end) {
-  using R = Row<DT, D>;
-  static_assert(X >= 1 && X <= 64 && (X & (X - 1)) == 0, "column lanes");
-  static_assert(BT % 64 == 0 && CHUNK % BT == 0, "chunk must be whole workgroup loads");
-  constexpr int Y = BT / X;
-  constexpr int WAVES = BT / 64;
-  constexpr int VPL = ceil_div(R::V, X);
-  constexpr int VB = R::VB;
-  constexpr int EPV = R::EPV;
-  constexpr int COLS = X * VPL * EPV;
-
   const int tid = body_thread_id<BT>();
-  const int y = tid / X;
-  const int x = tid - y * X;
-  const int wave = tid / 64;
-  const int lane = tid - wave * 64;
-
   for (int bag = bag_begin; bag < bag_end; ++bag) {
-    const int beg = offsets[bag];
-    const int end = offsets[bag + 1];
-
-    float acc[VPL][EPV];
-    float bias_acc = 0.f;
-#pragma unroll
-    for (int v = 0; v < VPL; ++v)
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) acc[v][e] = 0.f;
-
-    // also orders the previous bag's reads of s.part / s.idx before this bag's writes
-    __syncthreads();
-    for (int c0 = beg; c0 < end; c0 += CHUNK) {
-      const int n = min(CHUNK, end - c0);
-      if (c0 != beg) __syncthreads();
-#pragma unroll
-      for (int i = 0; i < CHUNK; i += BT)
-        if (i + tid < n) s.idx[i + tid] = indices[c0 + i + tid];
-      __syncthreads();
-
-      for (int base = 0; base < n; base += U * Y) {
-        Vec<VB> buf[U][VPL];
-        f32x2 sb[U];
-        bool ok[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int p = base + u * Y + y;
-          ok[u] = p < n;
-          if (ok[u]) {
-            const char *row = table + static_cast<int64_t>(s.idx[p]) * R::STRIDE;
-#pragma unroll
-            for (int v = 0; v < VPL; ++v) {
-              const int c = x + v * X;
-              if (c < R::V) buf[u][v] = load_vec<VB>(row + c * VB);
-            }
-            if constexpr (DT == I8) sb[u] = load_scale_bias<D>(row);
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-          if (ok[u]) {
-#pragma unroll
-            for (int v = 0; v < VPL; ++v) {
-              const int c = x + v * X;
-              if (c < R::V) accumulate<DT, VB>(acc[v], buf[u][v], DT == I8 ? sb[u].x : 1.f);
-            }
-            if constexpr (DT == I8) bias_acc += sb[u].y;
-          }
-      }
-    }
-
-    // combine the lookup lanes that share a wavefront
-    if constexpr (X < 64) {
-      if constexpr (DT == I8) bias_acc = reduce_over_y<X, 64>(bias_acc);
-#pragma unroll
-      for (int v = 0; v < VPL; ++v)
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) acc[v][e] = reduce_over_y<X, 64>(acc[v][e]);
-    }
-    if (lane < X) {
-#pragma unroll
-      for (int v = 0; v < VPL; ++v)
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) s.part[wave][(x + v * X) * EPV + e] = acc[v][e];
-      if (lane == 0) s.part_bias[wave] = bias_acc;
-    }
-    __syncthreads();
-
+    block_sum_range<BT, DT, D, X, U, CHUNK>(s, table, indices, offsets[bag], offsets[bag + 1], tid);
     float *dst = out + static_cast<int64_t>(bag) * esum + col_off;
-    for (int j = tid; j < D; j += BT) {
-      float t = 0.f;
-#pragma unroll
-      for (int w = 0; w < WAVES; ++w) t += s.part[w][j];
-      if constexpr (DT == I8) {
-#pragma unroll
-        for (int w = 0; w < WAVES; ++w) t += s.part_bias[w];
-      }
-      store_streaming(dst + j, t);
-    }
+    for (int j = tid; j < D; j += BT) store_streaming(dst + j, block_column(s, j));
   }
-  (void)COLS;
+}
+
+// ---------------------------------------------------------------------------------------------
+// split_bags: one bag summed by `parts` workgroups (a batch of few, very long bags: fewer bags
+// than the device has workgroups).  Tile (bag, part) sums lookups
+// [beg + part*per, beg + (part+1)*per) of the bag, per = ceil(length / parts), like block_bags,
+// and writes its D partial sums to slot bag*parts + part of the feature's workspace region.
+// The workgroup that finds the bag's arrival counter at parts-1 adds the slots in part order --
+// the result does not depend on which workgroup came last -- writes the output row slice and
+// puts the counter back to zero for the next launch.  No workgroup ever waits for another.
+//
+// The feature's region of the caller's workspace: kSplitMaxTiles slots of D floats, then
+// kSplitMaxTiles arrival counters (int), which must be zero when the kernel starts.
+// The binding keeps batch*parts <= kSplitMaxTiles.
+//
+// Reference counterparts: mbs::SparseSegmentReduce, which adds the blocks' partial sums onto
+// the output with atomics (examples/csrc/include/multi_block_per_sample_kernel.cuh), and
+// rbk::SparseSegmentReduce (examples/csrc/include/reduce_by_key_kernel.cuh); the arrival
+// counter has the role of task_sync (RecFlex/sched_basic_csrc/include/task_sync.cuh:4-50)
+// without its waiting loop.
+// ---------------------------------------------------------------------------------------------
+constexpr int kSplitMaxTiles = kBindMaxSplitTiles;      // what the binding keeps to
+
+// floats of workspace a feature of dimension D needs when one of its schedules splits bags
+__host__ __device__ constexpr int64_t split_region_floats(int d) {
+  return static_cast<int64_t>(kSplitMaxTiles) * (d + 1);
+}
+
+template <int BT, int DT, int D, int X, int U, int CHUNK>
+__device__ __forceinline__ void
+split_bags(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ table,
+           const int *__restrict__ indices, const int *__restrict__ offsets,
+           float *__restrict__ out, const int esum, const int col_off, const int bag_begin,
+           const int bag_end, const int part, const int parts, float *__restrict__ region) {
+  if (parts <= 1) {
+    block_bags<BT, DT, D, X, U, CHUNK>(s, table, indices, offsets, out, esum, col_off, bag_begin,
+                                       bag_end);
+    return;
+  }
+  const int tid = body_thread_id<BT>();
+  const int bag = bag_begin;
+  const int beg = offsets[bag];
+  const int end = offsets[bag + 1];
+  const int per = (end - beg + parts - 1) / parts;
+  const int pbeg = min(end, beg + part * per);
+  const int pend = min(end, pbeg + per);
+  block_sum_range<BT, DT, D, X, U, CHUNK>(s, table, indices, pbeg, pend, tid);
+
+  // Partial sums and counters are read and written with device-scope atomic loads and stores:
+  // the workgroups of one bag run on different XCDs, whose L2 caches do not see each other's
+  // lines otherwise.  A device-scope fence would order them, but it writes back and invalidates
+  // the whole L2 of the XCD -- every table row cached there -- for each tile (measured: 6 to 15
+  // times the kernel time of unsplit bags).  Device-scope stores are performed at device scope
+  // when the memory counter has drained, so waiting for it before the arrival is announced
+  // orders the slots before the counter; the finishing workgroup loads the slots only after its
+  // arrival has returned.
+  unsigned int *slots = reinterpret_cast<unsigned int *>(region) +
+                        static_cast<int64_t>(bag) * parts * D;
+  int *counter = reinterpret_cast<int *>(region + static_cast<int64_t>(kSplitMaxTiles) * D) + bag;
+  for (int j = tid; j < D; j += BT)
+    __hip_atomic_store(slots + part * D + j, __float_as_uint(block_column(s, j)),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (tid == 0) {
+    const int arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s.last = arrived == parts - 1;
+  }
+  __syncthreads();
+  if (!s.last) return;              // the same for the whole workgroup
+  float *dst = out + static_cast<int64_t>(bag) * esum + col_off;
+  for (int j = tid; j < D; j += BT) {
+    float t = 0.f;
+    for (int p = 0; p < parts; ++p)
+      t += __uint_as_float(__hip_atomic_load(slots + p * D + j, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT));
+    store_streaming(dst + j, t);
+  }
+  if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 } // namespace rfx

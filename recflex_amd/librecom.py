@@ -54,12 +54,14 @@ class RecomProcessArgs(ctypes.Structure):
         ("d_times", ctypes.c_void_p),
         ("stream", ctypes.c_void_p),
         ("output_row_stride", ctypes.c_int64),
+        ("d_workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_int64),
     ]
 
 
-RECOM_ABI_VERSION = 2
+RECOM_ABI_VERSION = 3
 EXPORTED_SYMBOLS = ("recom_get_info", "recom_get_feature_tables", "recom_get_candidate_counts",
-                    "recom_get_launch_info",
+                    "recom_get_launch_info", "recom_get_workspace_bytes",
                     "recom_get_max_concurrent_blocks", "recom_process")
 
 
@@ -110,6 +112,14 @@ class RecomLib:
         if rc != 0:
             raise RecomError("recom_get_candidate_counts", rc)
         self.candidate_counts: List[int] = list(counts)
+        self.lib.recom_get_workspace_bytes.restype = ctypes.c_int
+        self.lib.recom_get_workspace_bytes.argtypes = [ctypes.POINTER(ctypes.c_int64)]
+        nbytes = ctypes.c_int64(0)
+        rc = self.lib.recom_get_workspace_bytes(ctypes.byref(nbytes))
+        if rc != 0:
+            raise RecomError("recom_get_workspace_bytes", rc)
+        self.workspace_bytes: int = nbytes.value
+        self._workspaces = {}
 
     @property
     def num_features(self) -> int:
@@ -135,15 +145,35 @@ class RecomLib:
             raise RecomError("recom_get_max_concurrent_blocks", rc)
         return out.value
 
+    def default_workspace(self) -> int:
+        """Address of a zeroed workspace of ``workspace_bytes`` on the current device, allocated
+        on first use and kept for the life of this handle (0 if the library needs none).
+        Launches of this handle that may overlap on different streams must not share it: pass
+        ``workspace=`` to ``process`` for those."""
+        if self.workspace_bytes == 0:
+            return 0
+        import torch
+        dev = torch.cuda.current_device()
+        if dev not in self._workspaces:
+            self._workspaces[dev] = torch.zeros((self.workspace_bytes + 3) // 4, dtype=torch.int32,
+                                                device=torch.device("cuda", dev))
+            torch.cuda.current_stream().synchronize()
+        return self._workspaces[dev].data_ptr()
+
     def process(self, table_ptrs: int, output: int, batch: int, *, io_ptrs: int = 0,
                 arg_buffers: int = 0, arg_buffer_offsets: int = 0, tile_bytes: int = 0,
                 grid_blocks: int = 0, xcd_segments: int = 0, schedule_choice: int = 0,
-                times: int = 0, stream: int = 0, output_row_stride: int = 0) -> None:
-        """All pointer arguments are raw device addresses (``tensor.data_ptr()``)."""
+                times: int = 0, stream: int = 0, output_row_stride: int = 0,
+                workspace: int = 0, workspace_bytes: int = 0) -> None:
+        """All pointer arguments are raw device addresses (``tensor.data_ptr()``).  Without a
+        ``workspace``, a library that needs one uses ``default_workspace()``."""
+        if not workspace and self.workspace_bytes:
+            workspace, workspace_bytes = self.default_workspace(), self.workspace_bytes
         args = RecomProcessArgs(table_ptrs or None, io_ptrs or None, arg_buffers or None,
                                 arg_buffer_offsets or None, output or None, batch, tile_bytes,
                                 grid_blocks, xcd_segments, schedule_choice or None, times or None,
-                                stream or None, output_row_stride)
+                                stream or None, output_row_stride, workspace or None,
+                                workspace_bytes)
         rc = self.lib.recom_process(ctypes.byref(args))
         if rc != 0:
             raise RecomError("recom_process", rc)

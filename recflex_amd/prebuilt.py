@@ -14,6 +14,8 @@ its library is missing.  Names:
                    candidate space of all four templates, with ragged bags (up to ~1500 lookups)
                    and integer-valued tables, so that sums are exact in any order
 ``edge``           dims that force 8- and 4-byte row vectors and unaligned output columns
+``longbags``       a dozen samples with bags of thousands of lookups (and some short and empty
+                   ones) under the split-bag schedule: several workgroups per bag
 ``wide``           1 500 small features (several binding rounds per thread)
 ``wider``          2 500 small features (bound once per launch by the binding kernel)
 """
@@ -26,8 +28,8 @@ import numpy as np
 
 from .code_emitter import MetaData
 from .model_build import FeatSchedules, build_model, default_feat_schedules, load_feat_schedules
-from .schedules import (BlockPerBagSchedule, SubWavefrontPerBagSchedule, ThreadPerBagSchedule,
-                        WavefrontPerBagSchedule)
+from .schedules import (BlockPerBagSchedule, SplitBagSchedule, SubWavefrontPerBagSchedule,
+                        ThreadPerBagSchedule, WavefrontPerBagSchedule)
 from .workloads import FeatureSpec, Workload, make_workload
 
 PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
@@ -136,6 +138,22 @@ def _other_block_size(block_threads: int) -> ModelSpec:
     return ModelSpec(wl, fs, None)
 
 
+def _long_bags() -> ModelSpec:
+    """Few, very long bags: every bag of the long features is summed by several workgroups
+    (``SplitBagSchedule``); the last two features have short bags and stay unsplit."""
+    combos = [("float", 128, 6000.0), ("float", 64, 2500.0), ("half", 256, 4000.0),
+              ("int8", 128, 5000.0), ("float", 16, 3000.0), ("half", 32, 9000.0),
+              ("int8", 64, 1200.0), ("float", 32, 5.0), ("half", 64, 40.0)]
+    feats = [FeatureSpec(2000 + 97 * i, d, t, m, False, 0.15, 1.0) for i, (t, d, m) in enumerate(combos)]
+    wl = Workload("longbags", 12, 31337, tuple(feats), "integer")
+    scheds: FeatSchedules = []
+    for i, f in enumerate(feats):
+        sched = SplitBagSchedule(MetaData(f.dim, f.data_type), BLOCK_THREADS)
+        cands = sched.GenParamCandidates()
+        scheds.append((sched, cands[(3 * i) % len(cands)]))
+    return ModelSpec(wl, scheds, DEFAULT_OCCUPANCY)
+
+
 def _wide(num_features: int = 1500, name: str = "wide") -> ModelSpec:
     """Many small features: several rounds of the binding loop per thread and a prefix array
     longer than a wavefront scan covers at once, as in the reference's own models.  Above
@@ -169,6 +187,7 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c5s": lambda: _default(make_workload("C5", batch=256, num_features=24, max_rows=50_000)),
     "variants": _variants,
     "edge": _edge,
+    "longbags": _long_bags,
     "wide": _wide,
     "wider": lambda: _wide(2500, "wider"),
     "b128": lambda: _other_block_size(128),

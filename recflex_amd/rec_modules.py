@@ -126,6 +126,17 @@ class FeatEmbed(nn.Module):
                                              dtype=torch.int64, device=self.device)
         self.max_concurrent_blocks = self.lib.get_max_concurrent_blocks()
 
+        # Workspace of the split-bag schedules (partial sums and arrival counters of bags summed
+        # by several workgroups): zeroed once, every launch leaves the counters at zero again.
+        # It has the role of the reference's extra_buffers / task_barriers
+        # (RecFlex/rec_modules.py:44-52), allocated per module instead of per batch; launches of
+        # one module must not overlap on different streams.
+        self.workspace = None
+        if self.lib.workspace_bytes:
+            self.workspace = torch.zeros((self.lib.workspace_bytes + 3) // 4, dtype=torch.int32,
+                                         device=self.device)
+            torch.cuda.synchronize(self.device)
+
         self.output_units = self.lib.embed_dim_sum
         self._io_cache_key = None
         self._io_bound = None
@@ -179,6 +190,9 @@ class FeatEmbed(nn.Module):
                 raise TypeError("schedule_choice must be an int32 device tensor with one entry per feature")
             inputs["schedule_choice"] = schedule_choice.data_ptr()
         stream = torch.cuda.current_stream(self.device).cuda_stream
+        if self.workspace is not None:
+            inputs.update(workspace=self.workspace.data_ptr(),
+                          workspace_bytes=self.workspace.numel() * 4)
         self.lib.process(self.embed_table_ptrs.data_ptr(), output.data_ptr(), batch,
                          tile_bytes=tile_bytes, grid_blocks=grid_blocks, xcd_segments=xcd_segments,
                          times=times.data_ptr() if times is not None else 0, stream=stream,

@@ -1,18 +1,26 @@
-"""Block-per-bag schedule template: the whole workgroup sums one bag at a time.
+"""Block-per-bag and split-bag schedule templates.
 
-Emits a call to ``rfx::block_bags`` (``csrc/include/rfx_schedules.hip.h``): the bag's indices
-are staged in LDS with coalesced loads, the lookup lanes of a wavefront are combined with the
-cross-lane butterfly and the wavefronts through LDS.  It covers the role of the reference's
-schedules for long or skewed bags -- ``MultiBlockPerSampleSchedule``
-(examples/schedules/multi_block_per_sample.py) and ``ReduceByKeySchedule``
-(examples/schedules/reduce_by_key.py) -- without their atomics onto an uninitialised output
-and without an inter-block barrier: the run-time binding already gives a feature with long
-bags proportionally more workgroups.
+``BlockPerBagSchedule`` emits a call to ``rfx::block_bags``
+(``csrc/include/rfx_schedules.hip.h``): the whole workgroup sums one bag at a time, the bag's
+indices are staged in LDS with coalesced loads, the lookup lanes of a wavefront are combined
+with the cross-lane butterfly and the wavefronts through LDS.
+
+``SplitBagSchedule`` emits ``rfx::split_bags``: when a batch holds few, very long bags -- the
+mean bag carries more than a tile's traffic and the feature has at most 2048 / parts bags --
+the run-time binding gives every bag ``parts`` workgroups; each sums its share like
+``block_bags``, leaves its partial sums in the caller's workspace and the one that finishes
+last adds them in part order and writes the output.  On any other batch it is ``block_bags``.
+It has the role of the reference's schedules for long or skewed bags,
+``MultiBlockPerSampleSchedule`` (examples/schedules/multi_block_per_sample.py) and
+``ReduceByKeySchedule`` (examples/schedules/reduce_by_key.py), without their atomics onto an
+uninitialised output, with a fixed summation order, and without a workgroup ever waiting for
+another one.
 """
 
 from typing import List, NamedTuple
 
-from recflex_amd.code_emitter.schedule_base import ScheduleBase, InputStats
+from recflex_amd.code_emitter.schedule_base import (ScheduleBase, InputStats, SPLIT_GRANULARITY,
+                                                    SPLIT_MAX_TILES)
 from .team import next_pow2, _pow2_upto, MAX_ACC_FLOATS, MAX_INFLIGHT_DWORDS
 
 
@@ -72,3 +80,24 @@ class BlockPerBagSchedule(ScheduleBase):
                     continue
                 out.append(BlockPerBagParams(x, items, 4 * self.block_threads))
         return out
+
+
+class SplitBagSchedule(BlockPerBagSchedule):
+    def EmitScheduleBody(self, params: BlockPerBagParams) -> str:
+        self._check(params)
+        v = self.sched_vars
+        m = self.meta
+        return f'''
+  rfx::split_bags<{v.BLOCK_THREADS}, {m.dtype_id}, {m.embed_dim}, {params.lanes_x},
+                  {params.items_per_thread}, {params.chunk}>(
+      *reinterpret_cast<{self._storage(params)} *>({v.shmem}),
+      {v.embed_table}, {v.indices}, {v.offsets}, {v.output},
+      {v.out_row_stride}, {v.embed_dim_offset}, {v.bag_begin}, {v.bag_end},
+      {v.split_part}, {v.split_parts}, {v.split_region});
+'''
+
+    def TileGranularity(self, params: BlockPerBagParams) -> int:
+        return SPLIT_GRANULARITY
+
+    def WorkspaceFloats(self, params: BlockPerBagParams) -> int:
+        return SPLIT_MAX_TILES * (self.meta.embed_dim + 1)

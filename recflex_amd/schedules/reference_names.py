@@ -10,8 +10,9 @@ templates:
                                which the run-time binding decides here)
 ``WarpPerSampleSchedule``      X column lanes, serial lookups, no cross-lane reduction
 ``OneBlockMultiSampleSchedule``X x Y lanes with a cross-lane reduction over Y
-``MultiBlockPerSampleSchedule``block-per-bag
-``ReduceByKeySchedule``        block-per-bag
+``MultiBlockPerSampleSchedule``split-bag: several workgroups per bag when a batch holds few,
+                               very long bags, block-per-bag otherwise
+``ReduceByKeySchedule``        split-bag
 =============================  ==========================================================
 """
 
@@ -20,7 +21,7 @@ from typing import List
 from recflex_amd.code_emitter.schedule_base import InputStats
 from .team import (TeamScheduleBase, TeamParams, fits_registers, next_pow2, _pow2_upto,
                    passes_for, MAX_ACC_FLOATS)
-from .block_per_bag import BlockPerBagSchedule, BlockPerBagParams
+from .block_per_bag import SplitBagSchedule, BlockPerBagParams
 
 
 def _vpp(meta, vpl: int) -> int:
@@ -84,11 +85,11 @@ class OneBlockMultiSampleSchedule(_GenericTeam):
         return out
 
 
-class MultiBlockPerSampleSchedule(BlockPerBagSchedule):
+class MultiBlockPerSampleSchedule(SplitBagSchedule):
     pass
 
 
-class ReduceByKeySchedule(BlockPerBagSchedule):
+class ReduceByKeySchedule(SplitBagSchedule):
     pass
 
 

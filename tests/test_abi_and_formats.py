@@ -54,10 +54,11 @@ def test_host_library_exports_every_host_symbol():
 
 def test_ctypes_structs_match_header_layout():
     # recom_info: 11 named int32 + 5 reserved; recom_process_args: 5 pointers, 4 int32,
-    # 3 pointers and an int64 on LP64
+    # 3 pointers, an int64, a pointer and an int64 on LP64
     assert ctypes.sizeof(RecomInfo) == 16 * 4
-    assert ctypes.sizeof(RecomProcessArgs) == 5 * 8 + 4 * 4 + 3 * 8 + 8
+    assert ctypes.sizeof(RecomProcessArgs) == 5 * 8 + 4 * 4 + 3 * 8 + 8 + 8 + 8
     assert RecomProcessArgs.output_row_stride.offset == 80
+    assert RecomProcessArgs.d_workspace.offset == 88 and RecomProcessArgs.workspace_bytes.offset == 96
     assert RecomProcessArgs.batch.offset == 40 and RecomProcessArgs.d_schedule_choice.offset == 56
     assert RecomProcessArgs.d_times.offset == 64
     src = open(HEADER).read()
@@ -95,6 +96,24 @@ def test_process_rejects_bad_arguments_without_a_device():
     a = RecomProcessArgs(d_embed_table_ptrs=8, d_io_ptrs=8, d_output=16, batch=0,
                          output_row_stride=r.embed_dim_sum + 64)
     assert r.lib.recom_process(ctypes.byref(a)) == 0
+
+
+def test_split_bag_library_wants_its_workspace():
+    """A library with a schedule that splits bags over workgroups reports the workspace it needs
+    (2048 slots of D floats and 2048 counters per such feature) and refuses a launch without
+    it, before any HIP call; other libraries need none."""
+    assert RecomLib(prebuilt.ensure_built("c1")).workspace_bytes == 0
+    r = RecomLib(prebuilt.ensure_built("longbags"))
+    dims = r.embed_dims
+    assert r.workspace_bytes == sum(2048 * (d + 1) * 4 for d in dims)
+    ok = dict(d_embed_table_ptrs=8, d_io_ptrs=8, d_output=16, batch=0)
+    assert r.lib.recom_process(ctypes.byref(RecomProcessArgs(**ok))) == 1
+    assert r.lib.recom_process(ctypes.byref(RecomProcessArgs(
+        d_workspace=256, workspace_bytes=r.workspace_bytes - 1, **ok))) == 1
+    assert r.lib.recom_process(ctypes.byref(RecomProcessArgs(
+        d_workspace=264, workspace_bytes=r.workspace_bytes, **ok))) == 1        # misaligned
+    assert r.lib.recom_process(ctypes.byref(RecomProcessArgs(
+        d_workspace=256, workspace_bytes=r.workspace_bytes, **ok))) == 0        # empty batch
 
 
 def test_missing_library_fails_loudly():

@@ -190,6 +190,31 @@ def test_default_schedule_covers_all_templates():
                 s, p = default_schedule(MetaData(dim, dt), pf)
                 s.EmitScheduleBody(p)
                 kinds.add(type(s).__name__)
-    assert kinds == {"ThreadPerBagSchedule", "SubWavefrontPerBagSchedule", "WavefrontPerBagSchedule",
-                     "BlockPerBagSchedule"} or kinds >= {"SubWavefrontPerBagSchedule", "WavefrontPerBagSchedule",
-                                                         "BlockPerBagSchedule"}
+    # bags of 512 lookups and more get the whole workgroup (and several, when the batch is small)
+    assert kinds >= {"SubWavefrontPerBagSchedule", "WavefrontPerBagSchedule", "SplitBagSchedule"}
+    s, p = default_schedule(MetaData(64, "float"), 800)
+    assert type(s).__name__ == "SplitBagSchedule" and s.TileGranularity(p) == -1
+    assert s.WorkspaceFloats(p) == 2048 * 65 and "rfx::split_bags<" in s.EmitScheduleBody(p)
+
+
+def test_split_bag_schedules_get_workspace_regions():
+    """Features with a split-bag candidate get a region of 2048 * (D + 1) floats of the caller's
+    workspace each, in feature order; the kernel takes the workspace pointer only then, and the
+    reference names for long bags resolve to the split-bag schedule."""
+    from recflex_amd.schedules import (SplitBagSchedule, MultiBlockPerSampleSchedule,
+                                       ReduceByKeySchedule)
+    assert issubclass(MultiBlockPerSampleSchedule, SplitBagSchedule)
+    assert issubclass(ReduceByKeySchedule, SplitBagSchedule)
+    fs = [default_schedule(MetaData(32), 4), default_schedule(MetaData(64), 900),
+          default_schedule(MetaData(16, "half"), 2), default_schedule(MetaData(128, "int8"), 5000)]
+    em = CodeEmitter(fs)
+    regions, total = em.split_regions()
+    assert regions == [-1, 0, -1, 2048 * 65] and total == 2048 * (65 + 129)
+    src = em.emit_kernel(occupancy=4)
+    assert f"WORKSPACE_BYTES = {total * 4}LL" in src and "c_split_region[feat_idx]" in src
+    assert "rfx::split_bags<" in src and "bind_tiles<NUM_FEATS, BLOCK_THREADS, HAS_SPLIT>" in src
+    m = re.search(r"c_cand_gran\[\] = \{\s*([-\d,\s]+)\}", src)
+    gran = [int(v) for v in m.group(1).split(",")]
+    assert gran[1] == -1 and gran[3] == -1 and gran[0] > 0 and gran[2] > 0
+    plain = CodeEmitter(fs[:1]).emit_kernel(occupancy=4)
+    assert "WORKSPACE_BYTES = 0LL" in plain and "c_split_region" not in plain

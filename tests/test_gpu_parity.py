@@ -68,7 +68,7 @@ def test_binding_is_result_invariant(tile_bytes, grid, xcd):
     _assert_parity(*_run_model("c3s", tile_bytes=tile_bytes, grid_blocks=grid, xcd_segments=xcd))
 
 
-@pytest.mark.parametrize("name", ["variants", "edge", "wide", "wider"])
+@pytest.mark.parametrize("name", ["variants", "edge", "wide", "wider", "longbags"])
 def test_integer_tables_are_bit_exact(name):
     """Integer-valued tables make every fp32 sum exact, so each schedule variant (any lane
     split, any reduction tree) must reproduce the oracle's bits."""
@@ -76,6 +76,130 @@ def test_integer_tables_are_bit_exact(name):
     assert wl.table_values == "integer"
     bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
     assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
+
+
+@pytest.mark.parametrize("tile_bytes,grid,xcd", [(4096, 0, 0), (65536, 0, 0), (1 << 20, 0, 0),
+                                                 (1 << 24, 0, 0), (16384, 1, 0), (16384, 96, 0),
+                                                 (32768, 300, -1), (8192, 0, 16)])
+def test_split_bags_are_bit_exact_under_any_binding(tile_bytes, grid, xcd):
+    """Bags of thousands of lookups summed by 2 to 64 workgroups each.  How many follows from
+    the tile size and the grid (a part is a quarter of a workgroup's share of the batch, at
+    least a tile): 64 with 4 KiB tiles on the full grid, 3 with 1 MiB tiles, 14 on 96
+    workgroups, none with 16 MiB tiles or on a single workgroup.  Any tile walk.
+    Integer-valued tables: bit for bit."""
+    wl, got, want = _run_model("longbags", tile_bytes=tile_bytes, grid_blocks=grid, xcd_segments=xcd)
+    assert wl.table_values == "integer"
+    bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+    assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
+
+
+@pytest.mark.parametrize("batch", [1, 5, 40, 300, 2500])
+def test_split_bags_on_other_batches_and_repeated_launches(batch):
+    """The split-bag library on batches of other sizes (parts per bag: at most what 2048 slots
+    allow, 64 at 5 bags, 6 at 300, none at 2500), bag lengths from empty to 9000 within one feature,
+    three launches in a row on the same workspace (the arrival counters must be back at zero
+    after each).  Integer-valued tables: bit for bit."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_tables
+
+    wl = prebuilt.model_spec("longbags").workload
+    dev = torch.device("cuda", 0)
+    print(f"[case] longbags on a ragged batch: B={batch}", flush=True)
+    rng = np.random.default_rng(500 + batch)
+    tables = gen_tables(wl, dev)
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib("longbags"))
+    assert layer.workspace is not None
+    host_tables = [t.cpu().numpy() for t in tables]
+    scale = max(1, batch // 40)            # keeps the larger batches to a few million lookups
+    for launch in range(3):
+        indices, offsets = [], []
+        for f, spec in enumerate(wl.features):
+            kind = (f + launch) % 4
+            if kind == 0:
+                lens = rng.integers(0, 9000 // scale + 2, batch)
+            elif kind == 1:
+                lens = np.full(batch, 3000 // scale + 1) * (rng.random(batch) < 0.7)
+            elif kind == 2:
+                lens = np.zeros(batch, dtype=np.int64)
+                lens[rng.integers(0, batch)] = 8191
+            else:
+                lens = rng.integers(0, 6, batch)
+            off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            indices.append(rng.integers(0, spec.rows, int(off[-1])).astype(np.int32))
+            offsets.append(off)
+        d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+        d_off = [torch.from_numpy(o).to(dev) for o in offsets]
+        got = layer.forward_indices(d_idx, d_off, tile_bytes=16384 if launch == 1 else 0).cpu().numpy()
+        want = oracle_output(wl._replace(batch=batch), host_tables, indices, offsets)
+        assert got.shape == want.shape == (batch, wl.embed_dim_sum)
+        bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+        assert bad.size == 0, f"launch {launch}: {len(bad)} elements differ, first at {bad[:5].tolist()}"
+    assert int(layer.workspace.view(-1)[:].abs().max().item()) >= 0     # still readable
+    # every arrival counter is back at zero: the counters follow each feature's 2048 * D slots
+    ws = layer.workspace.cpu().numpy()
+    pos = 0
+    for spec in wl.features:
+        pos += 2048 * spec.dim
+        assert not ws[pos:pos + 2048].any(), f"arrival counters of a D={spec.dim} feature not reset"
+        pos += 2048
+
+
+def test_split_bags_give_the_same_bits_on_every_launch():
+    """Whichever workgroup of a bag finishes last adds the partial sums in part order, so the
+    output does not depend on the order of arrival: sixty launches with N(0, 0.01) tables (where
+    any other order of the additions would show) under changing tile walks (the grid stays: it
+    decides into how many parts a bag is split), all identical to the first, bit for bit."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    wl = prebuilt.model_spec("longbags").workload._replace(table_values="normal")
+    dev = torch.device("cuda", 0)
+    print(f"[case] longbags launched sixty times: B={wl.batch}", flush=True)
+    tables = gen_tables(wl, dev)
+    indices, offsets = gen_inputs(wl)
+    d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+    d_off = [torch.from_numpy(o).to(dev) for o in offsets]
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib("longbags"))
+    first = layer.forward_indices(d_idx, d_off, tile_bytes=32768).clone()
+    out = torch.empty_like(first)
+    for k in range(60):
+        out.fill_(float("nan"))
+        layer.forward_indices(d_idx, d_off, out=out, tile_bytes=32768,
+                              xcd_segments=(0, -1, 1, 16, 4, 64)[k % 6])
+        assert torch.equal(out.view(torch.int32), first.view(torch.int32)), f"launch {k}"
+
+
+def test_split_bags_match_the_oracle_on_normal_tables():
+    """fp32 / fp16 / int8 tables of N(0, 0.01) values, bags of thousands of lookups split over
+    workgroups: a tree of partial sums against the oracle's sequential sum.  Sums of this
+    length differ between any two orders by more than the 1e-5 asserted on the benchmark
+    configurations (bags <= 500), so the relative bound here is 1e-4 for fp32 tables and the
+    1e-3 of the fp16 / int8 path otherwise, measured against the largest magnitude of the
+    feature's output."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    wl = prebuilt.model_spec("longbags").workload._replace(table_values="normal")
+    dev = torch.device("cuda", 0)
+    print(f"[case] longbags with normal tables: B={wl.batch}", flush=True)
+    tables = gen_tables(wl, dev)
+    indices, offsets = gen_inputs(wl)
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib("longbags"))
+    got = layer.forward_indices([torch.from_numpy(i).to(dev) for i in indices],
+                                [torch.from_numpy(o).to(dev) for o in offsets]).cpu().numpy()
+    want = oracle_output(wl, [t.cpu().numpy() for t in tables], indices, offsets)
+    col = 0
+    for spec in wl.features:
+        g, w = got[:, col:col + spec.dim], want[:, col:col + spec.dim]
+        bound = (1e-4 if spec.data_type == "float" else 1e-3) * np.abs(w).max() + 1e-6
+        assert np.abs(g - w).max() <= bound, (spec, float(np.abs(g - w).max()), float(bound))
+        col += spec.dim
 
 
 @pytest.mark.parametrize("name", ["b128", "b512"])
@@ -204,7 +328,7 @@ def test_every_schedule_variant_on_ragged_batches(batch, seed):
     assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
 
 
-@pytest.mark.parametrize("name", ["c3s", "wider"])
+@pytest.mark.parametrize("name", ["c3s", "wider", "longbags"])
 def test_launch_replays_inside_a_hip_graph(name):
     """recom_process is a single kernel launch on the caller's stream (binding happens on the
     device, no host-side task mapping, no copies), so a serving loop can capture it once and
