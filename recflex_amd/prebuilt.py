@@ -16,6 +16,8 @@ its library is missing.  Names:
 ``edge``           dims that force 8- and 4-byte row vectors and unaligned output columns
 ``longbags``       a dozen samples with bags of thousands of lookups (and some short and empty
                    ones) under the split-bag schedule: several workgroups per bag
+``fewbags``        8 fp32 features x 16 samples x 20 000 lookups, default schedules (split-bag);
+                   ``fewbags_unsplit``: the same with one workgroup per bag, for comparison
 ``wide``           1 500 small features (several binding rounds per thread)
 ``wider``          2 500 small features (bound once per launch by the binding kernel)
 """
@@ -154,6 +156,18 @@ def _long_bags() -> ModelSpec:
     return ModelSpec(wl, scheds, DEFAULT_OCCUPANCY)
 
 
+def _few_bags(split: bool) -> ModelSpec:
+    """Fewer bags than the device has workgroups, each of 20 000 lookups."""
+    feats = tuple(FeatureSpec(2_000_000, d, "float", 20000.0, False, 0.0, 1.0)
+                  for d in (32, 64, 128, 64, 32, 128, 64, 64))
+    wl = Workload("fewbags", 16, 77, feats, "integer")
+    fs = default_feat_schedules(metas_of(wl), [f.mean_bag for f in feats], BLOCK_THREADS)
+    assert all(isinstance(s, SplitBagSchedule) for s, _ in fs)
+    if not split:
+        fs = [(BlockPerBagSchedule(s.meta, BLOCK_THREADS), p) for s, p in fs]
+    return ModelSpec(wl, fs, DEFAULT_OCCUPANCY)
+
+
 def _wide(num_features: int = 1500, name: str = "wide") -> ModelSpec:
     """Many small features: several rounds of the binding loop per thread and a prefix array
     longer than a wavefront scan covers at once, as in the reference's own models.  Above
@@ -188,6 +202,8 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "variants": _variants,
     "edge": _edge,
     "longbags": _long_bags,
+    "fewbags": lambda: _few_bags(True),
+    "fewbags_unsplit": lambda: _few_bags(False),
     "wide": _wide,
     "wider": lambda: _wide(2500, "wider"),
     "b128": lambda: _other_block_size(128),

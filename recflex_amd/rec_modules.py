@@ -246,6 +246,29 @@ class FeatEmbed(nn.Module):
         io_ptrs = torch.tensor(flat, dtype=torch.int64, device=self.device)
         return BoundInputs(batch, io_ptrs, (list(indices), list(offsets)))
 
+    def check_inputs(self, indices: Sequence[torch.Tensor], offsets: Sequence[torch.Tensor]) -> None:
+        """Debugging aid: raise ``ValueError`` if a launch on these inputs would read outside a
+        table or an index array -- offsets that do not start at 0, decrease, or end beyond the
+        index array; an index below 0 or beyond its table's rows.  The kernel itself checks
+        nothing (neither does the reference's), and an access outside device memory ends the
+        process.  Reads the inputs back with stock torch reductions and synchronises, so it is
+        meant for tests and for new data pipelines, not for the serving loop."""
+        self.bind_inputs(indices, offsets)              # types, shapes, devices
+        for f, (idx, off) in enumerate(zip(indices, offsets)):
+            rows = self.embed_tables[f].shape[0]
+            o = off.to(torch.int64)
+            if int(o[0]) != 0:
+                raise ValueError(f"feature {f}: offsets[0] = {int(o[0])}, expected 0")
+            if o.numel() > 1 and bool((o[1:] < o[:-1]).any()):
+                raise ValueError(f"feature {f}: offsets decrease")
+            used = int(o[-1])
+            if used > idx.numel():
+                raise ValueError(f"feature {f}: offsets end at {used}, beyond the {idx.numel()} indices")
+            if used > 0:
+                lo, hi = int(idx[:used].min()), int(idx[:used].max())
+                if lo < 0 or hi >= rows:
+                    raise ValueError(f"feature {f}: indices span [{lo}, {hi}], table has {rows} rows")
+
     def forward_indices(self, indices: Union["BoundInputs", Sequence[torch.Tensor]],
                         offsets: Sequence[torch.Tensor] = None,
                         timing: bool = False, timing_schedules: int = None, tile_bytes: int = 0,

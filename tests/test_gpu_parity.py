@@ -381,6 +381,38 @@ def test_launch_replays_inside_a_hip_graph(name):
         _assert_parity(wl, got.cpu().numpy(), want)
 
 
+def test_check_inputs_names_what_a_launch_would_trip_over():
+    """FeatEmbed.check_inputs accepts the generated batch and refuses, without launching
+    anything, offsets that decrease or overrun the index array and indices outside the table."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    wl = prebuilt.model_spec("c1").workload
+    dev = torch.device("cuda", 0)
+    print("[case] check_inputs on c1", flush=True)
+    tables = gen_tables(wl, dev)
+    indices, offsets = gen_inputs(wl)
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib("c1"))
+    d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+    d_off = [torch.from_numpy(o).to(dev) for o in offsets]
+    layer.check_inputs(d_idx, d_off)
+
+    def broken(which, f, pos, value):
+        idx, off = [t.clone() for t in d_idx], [t.clone() for t in d_off]
+        (idx if which == "idx" else off)[f][pos] = value
+        return idx, off
+
+    for args, what in ((("idx", 1, 7, wl.features[1].rows), "indices span"),
+                       (("idx", 2, 0, -1), "indices span"),
+                       (("off", 0, 5, 1 << 20), "offsets decrease"),
+                       (("off", 3, wl.batch, len(indices[3]) + 1), "beyond"),
+                       (("off", 0, 0, 1), "expected 0")):
+        with pytest.raises(ValueError, match=what):
+            layer.check_inputs(*broken(*args))
+
+
 def test_bound_inputs_give_the_same_output():
     """bind_inputs validates the tensors and uploads their addresses once; calls with its result
     skip the per-feature host work and must launch exactly what the list form launches, also
