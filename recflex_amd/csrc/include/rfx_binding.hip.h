@@ -53,14 +53,22 @@ struct IoView {
 // Schedules that split a bag over several workgroups (rfx::split_bags) announce themselves with
 // a granularity of kSplitGran.  A bag is worth splitting when it alone would keep its workgroup
 // busy for a good part of the kernel: the unit is a quarter of a workgroup's fair share of the
-// batch's traffic (total / grid), at least one tile; when the mean bag of such a feature
+// batch's traffic (total / grid), at least one tile and kSplitMinUnit; when the mean bag of such a feature
 // carries more than two units, the feature gets batch * parts tiles, parts = bag / unit, tile t
-// being part t % parts of bag t / parts, and bags_per_tile holds -parts;
-// parts <= kBindMaxParts and batch * parts <= kBindMaxSplitTiles (the slots of the feature's
+// being part t % parts of bag t / parts, and bags_per_tile holds -parts.  (A part costs some
+// 20 us of dependent memory round trips besides its rows, and with two to five tiles per
+// workgroup the time moves in steps of whole tiles: a unit of half a share gave 150 / 162 /
+// 161 us where a quarter gives 177 / 109 / 160 us on 16 x 20 000, 64 x 4 000 and 128 x 2 500
+// lookups; the finer one is kept, it also evens out bags of unequal length.)
+// Always parts <= kBindMaxParts and batch * parts <= kBindMaxSplitTiles (the slots of the feature's
 // workspace region).  Otherwise -- many bags, or a small grid -- the feature is bound like any
 // other with one bag per workgroup pass.  (Measured on 8 features of 16 bags of 20 000 lookups:
-// 968 us unsplit, 200 us split; 64 bags of 4 000: 204 and 105 us; 512 bags of 1 000 stay
+// 968 us unsplit, 177 us split; 64 bags of 4 000: 204 and 109 us; 512 bags of 1 000 stay
 // unsplit at 185 us.)
+// Smallest part: 256 KiB of traffic (with 128 KiB parts the three shapes above take 175 / 108 /
+// 161 us at four workgroups per CU, with 256 KiB parts 142 / 103 / 122 us; at eight workgroups
+// per CU, which these light kernels allow, 138 / 76 / 83 us and 107 / 83 / 96 us).
+constexpr int kSplitMinUnit = 256 * 1024;
 constexpr int kSplitGran = -1;
 constexpr int kBindMaxParts = 64;
 constexpr int kBindMaxSplitTiles = 2048;
@@ -198,6 +206,7 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     if (SPLIT) {
       split_unit = total / (4ll * (grid_blocks > 0 ? grid_blocks : 1));
       if (split_unit < tile_size) split_unit = tile_size;
+      if (split_unit < kSplitMinUnit) split_unit = kSplitMinUnit;
     }
     // the same decision in every thread of the grid
     if (SPLIT || tile_size != kAutoTileMin) {

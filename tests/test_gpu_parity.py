@@ -82,10 +82,10 @@ def test_integer_tables_are_bit_exact(name):
                                                  (1 << 24, 0, 0), (16384, 1, 0), (16384, 96, 0),
                                                  (32768, 300, -1), (8192, 0, 16)])
 def test_split_bags_are_bit_exact_under_any_binding(tile_bytes, grid, xcd):
-    """Bags of thousands of lookups summed by 2 to 64 workgroups each.  How many follows from
+    """Bags of thousands of lookups summed by several workgroups each.  How many follows from
     the tile size and the grid (a part is a quarter of a workgroup's share of the batch, at
-    least a tile): 64 with 4 KiB tiles on the full grid, 3 with 1 MiB tiles, 14 on 96
-    workgroups, none with 16 MiB tiles or on a single workgroup.  Any tile walk.
+    least a tile and 256 KiB): 12 for the longest bags on the full grid, 3 with 1 MiB tiles,
+    none with 16 MiB tiles or on a single workgroup.  Any tile walk.
     Integer-valued tables: bit for bit."""
     wl, got, want = _run_model("longbags", tile_bytes=tile_bytes, grid_blocks=grid, xcd_segments=xcd)
     assert wl.table_values == "integer"
@@ -96,7 +96,8 @@ def test_split_bags_are_bit_exact_under_any_binding(tile_bytes, grid, xcd):
 @pytest.mark.parametrize("batch", [1, 5, 40, 300, 2500])
 def test_split_bags_on_other_batches_and_repeated_launches(batch):
     """The split-bag library on batches of other sizes (parts per bag: at most what 2048 slots
-    allow, 64 at 5 bags, 6 at 300, none at 2500), bag lengths from empty to 9000 within one feature,
+    allow, 64 at 5 bags, 6 at 300, none at 2500), bag lengths from empty to 9000 within one
+    feature, a single bag of 40 000 lookups among empty ones (64 parts on a fp32 D=128 table),
     three launches in a row on the same workspace (the arrival counters must be back at zero
     after each).  Integer-valued tables: bit for bit."""
     import torch
@@ -123,7 +124,8 @@ def test_split_bags_on_other_batches_and_repeated_launches(batch):
                 lens = np.full(batch, 3000 // scale + 1) * (rng.random(batch) < 0.7)
             elif kind == 2:
                 lens = np.zeros(batch, dtype=np.int64)
-                lens[rng.integers(0, batch)] = 8191
+                # int8 sums stay exact in fp32 up to some ten thousand rows
+                lens[rng.integers(0, batch)] = 8191 if spec.data_type == "int8" else 40000
             else:
                 lens = rng.integers(0, 6, batch)
             off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
