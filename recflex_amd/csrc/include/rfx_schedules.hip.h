@@ -57,12 +57,114 @@ template <int BT> __device__ __forceinline__ int body_thread_id() {
 }
 
 // ---------------------------------------------------------------------------------------------
+// wave_bag: one bag summed by a whole wavefront, whatever the feature's schedule -- the way out
+// for a bag far longer than its feature's schedule was chosen for.  A team of T lanes with U
+// lookups in flight per lookup lane walks a bag of n lookups in n / (U*Y) dependent rounds of a
+// memory round trip each: a single bag of 2 000 lookups among one-lookup bags (16 lanes per bag,
+// one lookup in flight) held one wavefront for 1.2 ms in a kernel of 124 us, one of 20 000 for
+// 10 ms.  Here all 64 lanes work on the bag: as many column lanes as the row has vectors (at
+// most 64), the rest lookup lanes, four lookups in flight each (eight would push the
+// 100-feature kernel, which inlines this into twenty bodies, over its 96 registers: 8 spills),
+// indices fetched a round ahead, butterfly over the lookup lanes at the end.
+// No LDS and no barrier: only the wavefront that met the bag is involved.
+// ---------------------------------------------------------------------------------------------
+__host__ __device__ constexpr int pow2_at_least(int n) {
+  int p = 1;
+  while (p < n) p <<= 1;
+  return p;
+}
+
+template <int DT, int D, int OVEC>
+__device__ __forceinline__ void
+wave_bag(const char *__restrict__ table, const int *__restrict__ indices, const int beg,
+         const int end, float *__restrict__ dst, const int lane) {
+  using R = Row<DT, D>;
+  constexpr int XW = R::V >= 64 ? 64 : pow2_at_least(R::V);
+  constexpr int YW = 64 / XW;
+  constexpr int VPL = ceil_div(R::V, XW);
+  constexpr int VB = R::VB;
+  constexpr int EPV = R::EPV;
+  constexpr int UW = 4;
+
+  const int y = lane / XW;
+  const int x = lane - y * XW;
+  float acc[VPL][EPV];
+  float bias_acc = 0.f;
+#pragma unroll
+  for (int v = 0; v < VPL; ++v)
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) acc[v][e] = 0.f;
+
+  int idx[UW];
+#pragma unroll
+  for (int u = 0; u < UW; ++u) {
+    const int p = beg + u * YW + y;
+    idx[u] = p < end ? indices[p] : -1;
+  }
+  for (int base = beg; base < end; base += UW * YW) {
+    Vec<VB> buf[UW][VPL];
+    f32x2 sb[UW];
+#pragma unroll
+    for (int u = 0; u < UW; ++u)
+      if (idx[u] >= 0) {
+        const char *row = table + static_cast<int64_t>(idx[u]) * R::STRIDE;
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+          const int c = x + v * XW;
+          if (c < R::V) buf[u][v] = load_vec<VB>(row + c * VB);
+        }
+        if constexpr (DT == I8) sb[u] = load_scale_bias<D>(row);
+      }
+    int nidx[UW];
+#pragma unroll
+    for (int u = 0; u < UW; ++u) {
+      const int p = base + (UW + u) * YW + y;
+      nidx[u] = p < end ? indices[p] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < UW; ++u)
+      if (idx[u] >= 0) {
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+          const int c = x + v * XW;
+          if (c < R::V) accumulate<DT, VB>(acc[v], buf[u][v], DT == I8 ? sb[u].x : 1.f);
+        }
+        if constexpr (DT == I8) bias_acc += sb[u].y;
+      }
+#pragma unroll
+    for (int u = 0; u < UW; ++u) idx[u] = nidx[u];
+  }
+  if constexpr (XW < 64) {
+    if constexpr (DT == I8) bias_acc = reduce_over_y<XW, 64>(bias_acc);
+#pragma unroll
+    for (int v = 0; v < VPL; ++v)
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) acc[v][e] = reduce_over_y<XW, 64>(acc[v][e]);
+  }
+  if (y == 0) {
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+      const int c = x + v * XW;
+      if (c < R::V) {
+        if constexpr (DT == I8) {
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) acc[v][e] += bias_acc;
+        }
+        store_floats<EPV, OVEC>(dst + c * EPV, acc[v]);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // team_bags: teams of T <= 64 lanes; a workgroup of BT threads holds BT/T teams; team t sums
 // bags bag_begin + (t + k*TEAMS)*UB + [0, UB).
 //   U   lookups of one bag in flight per lookup lane
 //   UB  bags in flight per team (for short bags)
 //   VPP row vectors per lane per pass (a lane owns ceil(V/X) vectors; if that exceeds VPP the
 //       bag's index list is walked again for the next VPP vectors)
+// A bag of more than kLong = max(256, 16*U*Y) lookups (teams of fewer than 64 lanes) is not
+// walked by its team: the team's wavefront sums it with all its lanes first (wave_bag).
 // ---------------------------------------------------------------------------------------------
 template <int BT, int DT, int D, int X, int Y, int U, int UB, int VPP, int OVEC>
 __device__ __forceinline__ void
@@ -86,10 +188,16 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
   const int y = lt / X;
   const int x = lt - y * X;
 
-  for (int bag0 = bag_begin + team * UB; bag0 < bag_end; bag0 += TEAMS * UB) {
+  // Teams of fewer than 64 lanes: the wavefront stays together until its last team has run out
+  // of bags (teams beyond bag_end see empty bags), because a long bag needs all of its lanes.
+  auto more_bags = [&](const int bag0) {
+    if constexpr (T < 64) return __builtin_amdgcn_ballot_w64(bag0 < bag_end) != 0;
+    else return bag0 < bag_end;
+  };
+  for (int bag0 = bag_begin + team * UB; more_bags(bag0); bag0 += TEAMS * UB) {
     int beg[UB], end[UB];
     {
-      int prev = offsets[bag0];
+      int prev = offsets[bag0 < bag_end ? bag0 : bag_end];
 #pragma unroll
       for (int i = 0; i < UB; ++i) {
         const int b = bag0 + i + 1;
@@ -97,6 +205,29 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
         beg[i] = prev;
         end[i] = (bag0 + i < bag_end) ? next : prev;
         prev = next;
+      }
+    }
+    // bags far longer than this schedule suits: the whole wavefront sums them, one at a time;
+    // their teams then see an empty bag and leave the output alone
+    int done_mask = 0;
+    if constexpr (T < 64) {
+      constexpr int kLong = 16 * U * Y > 256 ? 16 * U * Y : 256;
+#pragma unroll
+      for (int i = 0; i < UB; ++i) {
+        const bool is_long = end[i] - beg[i] > kLong;
+        unsigned long long pending = __builtin_amdgcn_ballot_w64(is_long && lt == 0);
+        while (pending) {                         // the same in every lane of the wavefront
+          const int src = __builtin_ctzll(pending);
+          pending &= pending - 1;
+          const int b = __builtin_amdgcn_readlane(bag0 + i, src);
+          wave_bag<DT, D, OVEC>(table, indices, __builtin_amdgcn_readlane(beg[i], src),
+                                __builtin_amdgcn_readlane(end[i], src),
+                                out + static_cast<int64_t>(b) * esum + col_off, tid & 63);
+        }
+        if (is_long) {
+          done_mask |= 1 << i;
+          end[i] = beg[i];
+        }
       }
     }
     int len_max = 0;
@@ -246,7 +377,7 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
 #pragma unroll
         for (int i = 0; i < UB; ++i) {
           const int bag = bag0 + i;
-          const bool live = y == 0 && bag < bag_end;
+          const bool live = y == 0 && bag < bag_end && !((done_mask >> i) & 1);
           float *dst = out + static_cast<int64_t>(bag) * esum + col_off;
 #pragma unroll
           for (int v = 0; v < VPP; ++v) {
@@ -286,7 +417,7 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
 #pragma unroll
         for (int i = 0; i < UB; ++i) {
           const int bag = bag0 + i;
-          if (bag < bag_end) {
+          if (bag < bag_end && !((done_mask >> i) & 1)) {
             float *dst = out + static_cast<int64_t>(bag) * esum + col_off;
 #pragma unroll
             for (int v = 0; v < VPP; ++v) {

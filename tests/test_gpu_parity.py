@@ -311,7 +311,7 @@ def test_every_schedule_variant_on_ragged_batches(batch, seed):
             lens = rng.geometric(0.08, batch) * (rng.random(batch) < 0.6)  # heavy tail, 40 % empty
         elif kind == 2:
             lens = np.zeros(batch, dtype=np.int64)
-            lens[rng.integers(0, batch)] = 700                            # one long bag
+            lens[rng.integers(0, batch)] = 3000       # one outlier: summed by a whole wavefront
         elif kind == 3:
             lens = rng.integers(0, 4, batch)
         else:
