@@ -163,7 +163,7 @@ wave_bag(const char *__restrict__ table, const int *__restrict__ indices, const 
 //   UB  bags in flight per team (for short bags)
 //   VPP row vectors per lane per pass (a lane owns ceil(V/X) vectors; if that exceeds VPP the
 //       bag's index list is walked again for the next VPP vectors)
-// A bag of more than kLong = max(256, 16*U*Y) lookups (teams of fewer than 64 lanes) is not
+// A bag of more than kLong = max(64, 16*U*Y) lookups (teams of fewer than 64 lanes) is not
 // walked by its team: the team's wavefront sums it with all its lanes first (wave_bag).
 // ---------------------------------------------------------------------------------------------
 template <int BT, int DT, int D, int X, int Y, int U, int UB, int VPP, int OVEC>
@@ -211,7 +211,7 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
     // their teams then see an empty bag and leave the output alone
     int done_mask = 0;
     if constexpr (T < 64) {
-      constexpr int kLong = 16 * U * Y > 256 ? 16 * U * Y : 256;
+      constexpr int kLong = 16 * U * Y > 64 ? 16 * U * Y : 64;
 #pragma unroll
       for (int i = 0; i < UB; ++i) {
         const bool is_long = end[i] - beg[i] > kLong;
