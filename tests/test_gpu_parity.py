@@ -138,7 +138,6 @@ def test_split_bags_on_other_batches_and_repeated_launches(batch):
         assert got.shape == want.shape == (batch, wl.embed_dim_sum)
         bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
         assert bad.size == 0, f"launch {launch}: {len(bad)} elements differ, first at {bad[:5].tolist()}"
-    assert int(layer.workspace.view(-1)[:].abs().max().item()) >= 0     # still readable
     # every arrival counter is back at zero: the counters follow each feature's 2048 * D slots
     ws = layer.workspace.cpu().numpy()
     pos = 0
