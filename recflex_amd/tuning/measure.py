@@ -443,9 +443,11 @@ def auto_tile_bytes(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int],
 def tiles_per_feature(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int],
                       bag_bytes: Sequence[int], gran: Sequence[int], tile_bytes: int) -> List[int]:
     """Host restatement of the device binding (``rfx::bind_tiles``): tiles each feature gets
-    for this batch."""
+    for this batch.  A schedule that can split bags over workgroups (granularity -1) counts as
+    one bag per workgroup pass: a binding frozen at emit time never splits."""
     out = []
     for off, lb, bb, g in zip(offsets, lookup_bytes, bag_bytes, gran):
+        g = 1 if g < 0 else g
         batch = len(off) - 1
         if batch <= 0:
             out.append(0)
