@@ -55,7 +55,10 @@ typedef struct recom_info {
   int32_t static_binding; /* 1 if the tile count per feature was fixed at emit time */
   int32_t num_candidates; /* schedules compiled in; == num_features unless a tuning build */
   int32_t xcd_segments;   /* default of recom_process_args.xcd_segments (0 = flat tile walk) */
-  int32_t reserved[5];
+  int32_t outliers;       /* 1 if emitted with outlier tiles: recom_process first launches a kernel
+                           * that lists the bags too long for their feature's schedule, and the
+                           * fused kernel runs them as tiles of their own, several workgroups each */
+  int32_t reserved[4];
 } recom_info;
 
 #define RECOM_ABI_VERSION 3     /* 3: recom_get_workspace_bytes, d_workspace / workspace_bytes */
@@ -86,8 +89,10 @@ int recom_get_max_concurrent_blocks(int32_t *out);
 
 /* Bytes of recom_process_args.d_workspace this library needs: 0 unless a feature runs a
  * schedule that splits bags over workgroups, then 2048 * (D_f + 1) * 4 bytes for each such
- * feature (rounded up to 128).  Replaces the extra-buffer sizes the reference's host
- * preprocessors report per batch (RecFlex/code_emitter/codegen.py:149-160, extra_buffer_offsets). */
+ * feature (rounded up to 128); a library with outlier tiles adds its list of outliers and
+ * their partial sums (26 752 + 16 384 * max dim bytes).  Replaces the extra-buffer sizes the
+ * reference's host preprocessors report per batch (RecFlex/code_emitter/codegen.py:149-160,
+ * extra_buffer_offsets). */
 int recom_get_workspace_bytes(int64_t *out);
 
 typedef struct recom_launch_info {
@@ -166,7 +171,9 @@ typedef struct recom_process_args {
  *   output[b, off_f : off_f + D_f] = sum_{p in [offsets_f[b], offsets_f[b+1])} row(table_f, indices_f[p])
  * Asynchronous.  Replaces torch.ops.recom.process (RecFlex/code_emitter/codegen.py:403-444)
  * and FusedKnl (RecFlex/code_emitter/codegen.py:318-383).
- * Never allocates.  A library of more than 2048 features launches a one-workgroup kernel ahead
+ * Never allocates.  A library emitted with outlier tiles (recom_info.outliers) launches a small
+ * kernel ahead that walks the offsets and lists the outlier bags in the workspace.
+ * A library of more than 2048 features launches a one-workgroup kernel ahead
  * of the fused one that binds the model for this batch into a static device array of the
  * library; the array has one slot per stream (eight), launches on one stream share theirs, and
  * a ninth stream on the same device is refused with hipErrorOutOfMemory (2). */

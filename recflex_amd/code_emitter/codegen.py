@@ -40,6 +40,8 @@ LOOKUP_OVERHEAD_BYTES = 0
 # models of more features than this are bound once per launch by a small kernel instead of by
 # every workgroup of the fused kernel (rfx::bind_once)
 BIND_ONCE_MIN_FEATS = 2048
+# a bag becomes tiles of its own (libraries emitted with outliers=True) from this much traffic
+OUTLIER_MIN_BYTES = 128 * 1024
 
 
 def _c_array(ctype: str, name: str, values: List[int], per_line: int = 16) -> str:
@@ -130,6 +132,31 @@ class CodeEmitter:
             total += need
         return regions, total
 
+    def long_bag_tables(self) -> Tuple[List[int], List[Tuple[int, int]], List[int]]:
+        """For a build with outlier tiles: per feature the bag length beyond which a bag is run
+        as tiles of its own (beyond its schedule's threshold and carrying at least
+        OUTLIER_MIN_BYTES of traffic; 0 = none), the distinct
+        (element type, dim) pairs of the features that have one, and per feature the index of
+        its pair (-1 = none)."""
+        thr, keys, body_of = [], [], []
+        for cands in self.feat_candidates:
+            t = [schedule.LongBagThreshold(params) for schedule, params in cands]
+            t = 0 if min(t) <= 0 else max(t)
+            if t > 0:
+                per_lookup = cands[0][0].meta.row_bytes + INDEX_BYTES
+                t = max(t, -(-OUTLIER_MIN_BYTES // per_lookup))
+            thr.append(t)
+            key = (cands[0][0].meta.dtype_id, cands[0][0].meta.embed_dim)
+            if t > 0 and key not in keys:
+                keys.append(key)
+            body_of.append(keys.index(key) if t > 0 else -1)
+        return thr, keys, body_of
+
+    @staticmethod
+    def _meta_of(dtype_id: int, dim: int):
+        from .schedule_base import MetaData
+        return MetaData(dim, ("float", "half", "int8")[dtype_id])
+
     def dedup(self) -> Tuple[Dict[int, int], List[int]]:
         """candidate index -> index of the first candidate with the same (LDS type, body); list
         of those first indices.  With one schedule per feature, candidate index == feature."""
@@ -147,7 +174,7 @@ class CodeEmitter:
 
     def emit_headers(self) -> str:
         headers = {"<hip/hip_runtime.h>", "<stdint.h>", '"recflex_hip.h"', '"rfx_binding.hip.h"',
-                   '"rfx_launch.hip.h"'}
+                   '"rfx_launch.hip.h"', '"rfx_outliers.hip.h"', '"rfx_schedules.hip.h"'}
         for schedule, params in self.feat_schedules:
             headers = headers.union(schedule.EmitHeaders())
         return ''.join(sorted(f"#include {header}\n" for header in headers)) + '\n'
@@ -155,7 +182,8 @@ class CodeEmitter:
     def emit_kernel(self, occupancy: int = None, inline: bool = True, timing: bool = False,
                     timing_branch: bool = False, fixed_task_block_nums: List[int] = None,
                     tile_bytes: int = None, xcd_aware: bool = False,
-                    lookup_overhead_bytes: int = None, xcd_segments: int = 8) -> str:
+                    lookup_overhead_bytes: int = None, xcd_segments: int = 8,
+                    outliers: bool = False) -> str:
         num_feats = len(self.feat_schedules)
         if lookup_overhead_bytes is None:
             lookup_overhead_bytes = LOOKUP_OVERHEAD_BYTES
@@ -167,6 +195,14 @@ class CodeEmitter:
         bind_once = num_feats > BIND_ONCE_MIN_FEATS
         split_regions, workspace_floats = self.split_regions()
         has_split = workspace_floats > 0
+        assert not (outliers and (timing or fixed_task_block_nums)), \
+            "outlier tiles are for production builds (no per-feature timers, no frozen binding)"
+        # the list of outliers is made with one threshold per feature, which the feature's body
+        # must share: one schedule per feature
+        assert not outliers or all(len(c) == 1 for c in self.feat_candidates)
+        long_thr, long_keys, long_body_of = self.long_bag_tables() if outliers else ([], [], [])
+        outliers = outliers and len(long_keys) > 0
+        max_long_dim = max([(d + 3) // 4 * 4 for _, d in long_keys], default=4)
         fixed_arg = "c_fixed_task_block_nums" if fixed_task_block_nums else "nullptr"
 
         consts = f'''constexpr int NUM_FEATS = {num_feats};
@@ -184,8 +220,14 @@ constexpr bool STATIC_BINDING = {"true" if fixed_task_block_nums else "false"};
 #define RFX_BIND_ONCE {1 if bind_once else 0}
 constexpr bool BIND_ONCE = RFX_BIND_ONCE;
 // bytes of caller workspace the split-bag schedules need (0: no schedule splits bags)
-constexpr long long WORKSPACE_BYTES = {workspace_floats * 4}LL;
-constexpr bool HAS_SPLIT = WORKSPACE_BYTES > 0;
+constexpr long long SPLIT_BYTES = {workspace_floats * 4}LL;
+constexpr bool HAS_SPLIT = SPLIT_BYTES > 0;
+// outlier bags found ahead of the kernel and run as tiles of their own (rfx_outliers.hip.h)
+#define RFX_OUTLIERS {1 if outliers else 0}
+constexpr bool OUTLIERS = RFX_OUTLIERS;
+constexpr int MAX_LONG_DIM = {max_long_dim};
+using OutlierSpace = rfx::OutlierSpace<MAX_LONG_DIM>;
+constexpr long long WORKSPACE_BYTES = SPLIT_BYTES + (OUTLIERS ? (long long)sizeof(OutlierSpace) : 0LL);
 static_assert(rfx::kBindMaxSplitTiles == {SPLIT_MAX_TILES} && rfx::kSplitGran == {SPLIT_GRANULARITY},
               "workspace regions were sized for this");
 
@@ -207,9 +249,25 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
     const int {vars_.bag_begin}, const int {vars_.bag_end},
     char *__restrict__ {vars_.shmem}, rfx::f32x4 *__restrict__ {vars_.stage},
     const int {vars_.split_part}, const int {vars_.split_parts},
-    float *__restrict__ {vars_.split_region}) {{
+    float *__restrict__ {vars_.split_region}, const int {vars_.skip_long}) {{
   {schedule.EmitScheduleBody(params)}
 }}
+'''
+        # one block-wide body per (element type, dim) that can have outliers
+        long_cases = ""
+        for k, (dtype_id, dim) in enumerate(long_keys):
+            meta = self._meta_of(dtype_id, dim)
+            lanes = min(64, 1 << (meta.row_vectors - 1).bit_length())
+            items = 4 if meta.elems_per_vector <= 4 else 2
+            storage = (f"rfx::BlockBagStorage<{vars_.BLOCK_THREADS}, {dtype_id}, {dim}, {lanes}, "
+                       f"{4 * self.block_threads}>")
+            temp_storage_decl += f"  {storage} long{k};\n"
+            long_cases += f'''        case {k}:
+          rfx::split_part<{vars_.BLOCK_THREADS}, {dtype_id}, {dim}, {lanes}, {items}, {4 * self.block_threads}>(
+              *reinterpret_cast<{storage} *>(&s), table, indices, offsets, d_output,
+              {vars_.out_row_stride}, embed_dim_offset, e.bag, part, e.parts,
+              &d_outliers->slots[e.first][0], MAX_LONG_DIM, &d_outliers->counters[entry]);
+          break;
 '''
         temp_storage_decl += "};\n\n"
 
@@ -225,6 +283,9 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
         if has_split:
             # first float of each feature's region of the workspace (-1: the feature has none)
             tables += _c_array("long long", "c_split_region", split_regions)
+        if outliers:
+            tables += _c_array("int", "c_long_thr", long_thr)
+            tables += _c_array("int", "c_long_body", long_body_of)
         if fixed_task_block_nums:
             assert len(fixed_task_block_nums) == num_feats
             tables += _c_array("int", "c_fixed_task_block_nums",
@@ -265,7 +326,7 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
         call_args = (f"table, indices, offsets, d_output, {vars_.out_row_stride}, embed_dim_offset, "
                      f"{vars_.bag_begin}, {vars_.bag_end}, reinterpret_cast<char *>(&s), "
                      + ("&s_stage.seg[0][0]" if need_stage else "nullptr")
-                     + f", {vars_.split_part}, {vars_.split_parts}, {vars_.split_region}")
+                     + f", {vars_.split_part}, {vars_.split_parts}, {vars_.split_region}, {vars_.skip_long}")
         cases = "".join(
             f"      case {feat_idx}: ProcessFeat{feat_idx}({call_args}); break;\n"
             for feat_idx in body_ids)
@@ -274,12 +335,12 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
                          else f"__launch_bounds__({vars_.BLOCK_THREADS})")
         if bind_once:
             bind_decl = "  __shared__ rfx::PrefixStorage<NUM_FEATS> s_bind;\n"
-            bind_call = (f"  const int total_tiles = rfx::load_prefix<NUM_FEATS, {vars_.BLOCK_THREADS}>"
+            bind_call = (f"  const int regular_tiles = rfx::load_prefix<NUM_FEATS, {vars_.BLOCK_THREADS}>"
                          "(s_bind, d_bound);\n  (void)tile_bytes;\n  (void)d_schedule_choice;")
             bound_src = "d_bound->"
         else:
             bind_decl = "  __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;\n"
-            bind_call = (f"  const int total_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}, HAS_SPLIT>(\n"
+            bind_call = (f"  const int regular_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}, HAS_SPLIT>(\n"
                          "      s_bind, io, tile_bytes, c_lookup_bytes, c_bag_bytes, c_cand_begin, c_cand_gran,\n"
                          f"      d_schedule_choice, {fixed_arg}, gridDim.x);\n  (void)d_bound;")
             bound_src = "s_bind."
@@ -304,7 +365,46 @@ extern "C" __global__ void __launch_bounds__(1024) BindKnl(
 static __device__ __align__(256) char g_bound[256];     // unused: every workgroup binds for itself
 '''
 
-        kernel = bind_kernel + f'''
+        outlier_kernel = '''
+// Finds the bags that are too long for their feature's schedule (one thread per bag).
+extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
+    const int64_t *__restrict__ d_io_ptrs, const char *__restrict__ d_arg_buffers,
+    const int64_t *__restrict__ d_arg_buffer_offsets, const int batch,
+    OutlierSpace *__restrict__ d_outliers) {
+  const rfx::IoView io{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch};
+  rfx::find_outliers<NUM_FEATS, MAX_LONG_DIM>(d_outliers, io, c_long_thr, c_lookup_bytes);
+}
+''' if outliers else ''
+        outlier_begin = '''
+  // outlier parts come first in the tile space: they are the longest tiles
+  const int outlier_tiles = rfx::outlier_parts(d_outliers);
+  const int total_tiles = regular_tiles + outlier_tiles;
+''' if outliers else '''
+  constexpr int outlier_tiles = 0;
+  const int total_tiles = regular_tiles;
+  (void)d_outliers;
+'''
+        outlier_tile = f'''
+    if (tile < outlier_tiles) {{
+      const int entry = d_outliers->partmap[tile];
+      const rfx::OutlierEntry e = d_outliers->entries[entry];
+      const int part = tile - e.first;
+      const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[e.feat]);
+      const int *indices = io.indices(e.feat);
+      const int *offsets = io.offsets(e.feat);
+      const int embed_dim_offset = c_embed_dim_offsets[e.feat];
+      switch (c_long_body[e.feat]) {{
+{long_cases}        default: break;
+      }}
+      continue;
+    }}
+    tile -= outlier_tiles;
+''' if outliers else ''
+        outlier_end = '''
+  __syncthreads();
+  if (threadIdx.x == 0) rfx::outliers_done(d_outliers);
+''' if outliers else ''
+        kernel = bind_kernel + outlier_kernel + f'''
 extern "C" __global__ void {launch_bounds} FusedKnl(
     const int64_t *__restrict__ d_embed_table_ptrs,
     const int64_t *__restrict__ d_io_ptrs,
@@ -314,13 +414,15 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     const int batch, const int tile_bytes, const int xcd_segments,
     const int *__restrict__ d_schedule_choice,
     unsigned long long *__restrict__ d_times, const int {vars_.out_row_stride},
-    const rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound, float *__restrict__ d_workspace) {{
+    const rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound, float *__restrict__ d_workspace,
+    OutlierSpace *__restrict__ d_outliers) {{
 {bind_decl}
   __shared__ KnlTempStorage s;
 {stage_decl}{timing_init}
   const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
 {bind_call}
 
+{outlier_begin}
   // Tiles are ordered by feature.  Workgroup i runs on XCD i % XCDS.  With xcd_segments > 0 the
   // tile space is cut into XCDS * xcd_segments equal segments and segment s belongs to XCD
   // s % XCDS: a feature's tiles
@@ -343,7 +445,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
       tile = (seg * XCDS + xcd) * seg_len + (walk - seg * seg_len);
       if (tile >= total_tiles) continue;
     }}
-{timing_begin if timing and timing_branch else ''}
+{outlier_tile}{timing_begin if timing and timing_branch else ''}
     const int feat_idx = __builtin_amdgcn_readfirstlane(rfx::find_feature<NUM_FEATS>(s_bind.prefix, tile));
     const int bags_per_tile = {bound_src}bags_per_tile[feat_idx];
     int {vars_.bag_begin} = (tile - s_bind.prefix[feat_idx]) * bags_per_tile;
@@ -366,13 +468,14 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     const int *indices = io.indices(feat_idx);
     const int *offsets = io.offsets(feat_idx);
     const int embed_dim_offset = c_embed_dim_offsets[feat_idx];
+    const int {vars_.skip_long} = {"outlier_tiles > 0 && c_long_thr[feat_idx] > 0 ? c_long_thr[feat_idx] : 0x7fffffff" if outliers else "0x7fffffff"};
 {timing_begin if timing and not timing_branch else ''}
     switch (c_cand_func_ids[{bound_src}cand[feat_idx]]) {{
 {cases}      default: break;
     }}
 {timing_end}
   }}
-{timing_flush}}}
+{timing_flush}{outlier_end}}}
 
 '''
         return consts + temp_storage_decl + functions + "\n" + tables + kernel
@@ -392,7 +495,7 @@ extern "C" int recom_process(const recom_process_args *a) {
       reinterpret_cast<uintptr_t>(a->d_output) % (OUT_VEC * sizeof(float)) != 0)
     return static_cast<int>(hipErrorInvalidValue);
   // split-bag schedules keep partial sums and arrival counters in the caller's workspace
-  if (HAS_SPLIT && (!a->d_workspace || a->workspace_bytes < WORKSPACE_BYTES ||
+  if (WORKSPACE_BYTES > 0 && (!a->d_workspace || a->workspace_bytes < WORKSPACE_BYTES ||
                     reinterpret_cast<uintptr_t>(a->d_workspace) % 16 != 0))
     return static_cast<int>(hipErrorInvalidValue);
   if (a->batch == 0) return static_cast<int>(hipSuccess);
@@ -412,7 +515,19 @@ extern "C" int recom_process(const recom_process_args *a) {
   int batch = a->batch, tile_arg = tile_bytes, xcd_arg = xcd_segments;
   int stride_arg = static_cast<int>(row_stride);
   void *workspace = a->d_workspace;
+  void *outlier_space = OUTLIERS ? static_cast<char *>(a->d_workspace) + SPLIT_BYTES : nullptr;
   void *bound = nullptr;
+#if RFX_OUTLIERS
+  {
+    void *outlier_args[] = {const_cast<int64_t **>(&a->d_io_ptrs), &arg_buffers,
+                            const_cast<int64_t **>(&a->d_arg_buffer_offsets), &batch, &outlier_space};
+    const unsigned gx = static_cast<unsigned>((batch + 255) / 256 > 64 ? 64 : (batch + 255) / 256);
+    const unsigned gy = static_cast<unsigned>(NUM_FEATS > 1024 ? 1024 : NUM_FEATS);
+    e = hipLaunchKernel(reinterpret_cast<const void *>(OutlierKnl), dim3(gx, gy), dim3(256),
+                        outlier_args, 0, static_cast<hipStream_t>(a->stream));
+    if (e != hipSuccess) return static_cast<int>(e);
+  }
+#endif
 #if RFX_BIND_ONCE
   e = rfx::bind_slot_for(
       [](char **p) {
@@ -434,7 +549,8 @@ extern "C" int recom_process(const recom_process_args *a) {
       &arg_buffers, const_cast<int64_t **>(&a->d_arg_buffer_offsets),
       const_cast<float **>(&a->d_output), &batch, &tile_arg, &xcd_arg,
       const_cast<int32_t **>(&a->d_schedule_choice),
-      const_cast<unsigned long long **>(&a->d_times), &stride_arg, &bound, &workspace};
+      const_cast<unsigned long long **>(&a->d_times), &stride_arg, &bound, &workspace,
+      &outlier_space};
   e = hipLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
                       kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream));
   return static_cast<int>(e);
@@ -492,6 +608,7 @@ extern "C" int recom_get_info(recom_info *out) {
   out->static_binding = STATIC_BINDING ? 1 : 0;
   out->num_candidates = NUM_CANDIDATES;
   out->xcd_segments = XCD_SEGMENTS;
+  out->outliers = OUTLIERS ? 1 : 0;
   return 0;
 }
 
@@ -541,7 +658,7 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
              tune: bool = False, timing: bool = False, timing_branch: bool = False,
              fixed_task_block_nums: List[int] = None, tile_bytes: int = None,
              xcd_aware: bool = False, lookup_overhead_bytes: int = None,
-             xcd_segments: int = 8) -> None:
+             xcd_segments: int = 8, outliers: bool = False) -> None:
         """Write the device source.  ``occupancy`` = workgroups per CU the kernel is built and
         launched for (``__launch_bounds__`` budget, persistent grid size, and a dynamic-LDS pad
         that keeps further workgroups off the CU); ``tune`` is accepted for signature
@@ -553,7 +670,7 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
                                  fixed_task_block_nums=fixed_task_block_nums,
                                  tile_bytes=tile_bytes, xcd_aware=xcd_aware,
                                  lookup_overhead_bytes=lookup_overhead_bytes,
-                                 xcd_segments=xcd_segments)
+                                 xcd_segments=xcd_segments, outliers=outliers)
         code += self.emit_process_func(timing=timing, occupancy=occupancy)
         code += self.emit_get_concurrent_blocks_func(occupancy=occupancy)
         code += self.emit_process_ops()

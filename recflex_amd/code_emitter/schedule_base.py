@@ -112,6 +112,9 @@ class ScheduleVars(NamedTuple):
     # schedules that split a bag over workgroups: this tile is part split_part of split_parts of
     # bag bag_begin (split_parts <= 1: a plain bag range); split_region = the feature's floats
     # of the caller's workspace (null if no schedule of the feature splits)
+    # int: bags of more lookups than this were found ahead of the kernel and run as tiles of
+    # their own, the body must leave them alone (INT_MAX when there are none)
+    skip_long: str = "skip_longer_than"
     split_part: str = "split_part"
     split_parts: str = "split_parts"
     split_region: str = "split_region"
@@ -150,6 +153,13 @@ class ScheduleBase(ABC):
     @abstractmethod
     def TileGranularity(self, params: NamedTuple) -> int:
         """Bags one workgroup of this schedule covers per pass; tiles are multiples of it."""
+
+    def LongBagThreshold(self, params: NamedTuple) -> int:
+        """Bags of more lookups than this are outliers for the schedule.  A library emitted with
+        ``outliers=True`` gives those of them that carry at least a tile's traffic to several
+        workgroups and tells the body which to skip (``skip_long``).  0: the schedule takes bags
+        of any length and ignores that."""
+        return 0
 
     def WorkspaceFloats(self, params: NamedTuple) -> int:
         """Floats of the caller's workspace this schedule needs for its feature (0 = none).  A

@@ -1,0 +1,100 @@
+// Outlier bags given to many workgroups (optional part of the fused embedding kernel, for data
+// whose bag lengths are skewed).
+//
+// A bag far longer than its feature's schedule was chosen for keeps one team -- at best one
+// wavefront (rfx::wave_bag) -- busy long after the rest of the grid has finished.  A library
+// emitted with outliers=True launches find_outliers ahead of the fused kernel: it walks all
+// offsets of the batch, and every bag longer than its schedule's threshold
+// (rfx::long_bag_threshold) becomes an entry {feature, bag, first part, parts} of a list in the
+// caller's workspace, parts = its traffic / kOutlierUnit (1..kOutlierMaxParts).  The fused
+// kernel runs the parts of all entries as its first tiles, each like a part of a split bag
+// (rfx::split_part: partial sums in a slot, arrival counter, the last one adds the slots in
+// part order and writes the output), and its teams leave those bags alone.  If the list
+// overflows (more than kOutlierCap bags or kOutlierPartCap parts) the launch falls back to the
+// wavefront path for all of them.  The workgroup that finishes last puts the list header back
+// to zero for the next launch.
+//
+// Reference counterpart: the role of rbk::SparseSegmentReduce
+// (examples/csrc/include/reduce_by_key_kernel.cuh), load balance under skewed bag lengths.
+#pragma once
+#include "rfx_binding.hip.h"
+
+namespace rfx {
+
+constexpr int kOutlierCap = 512;             // entries
+constexpr int kOutlierPartCap = 4096;        // parts of all entries together
+constexpr int kOutlierUnit = 128 * 1024;     // traffic of one part
+constexpr int kOutlierMaxParts = 64;
+
+struct OutlierHeader {
+  unsigned long long pack;                   // entries << 32 | parts, both as reserved so far
+  int finished;                              // workgroups of the fused kernel that are done
+  int last_entries, last_parts;              // what the previous launch found (for the caller)
+  int pad[27];
+};
+struct OutlierEntry {
+  int feat, bag, first, parts;
+};
+
+// MAXD: largest embedding dimension among the features that can have outliers, rounded up to 4
+template <int MAXD> struct OutlierSpace {
+  OutlierHeader hdr;
+  OutlierEntry entries[kOutlierCap];
+  int counters[kOutlierCap];                 // arrival counters, zero between launches
+  int partmap[kOutlierPartCap];              // part -> entry
+  unsigned int slots[kOutlierPartCap][MAXD]; // partial sums
+};
+
+// One thread per (feature, bag); grid (x: bags, y: features), any size.
+template <int F, int MAXD>
+__device__ __forceinline__ void
+find_outliers(OutlierSpace<MAXD> *__restrict__ sp, const IoView &io,
+              const int *__restrict__ long_thr, const int *__restrict__ lookup_bytes) {
+  for (int f = blockIdx.y; f < F; f += gridDim.y) {
+    const int thr = long_thr[f];
+    if (thr <= 0) continue;                  // a schedule that handles long bags itself
+    const int *offs = io.offsets(f);
+    for (int b = blockIdx.x * blockDim.x + threadIdx.x; b < io.batch; b += gridDim.x * blockDim.x) {
+      const int len = offs[b + 1] - offs[b];
+      if (len <= thr) continue;
+      const long long cost = static_cast<long long>(len) * lookup_bytes[f];
+      long long want = (cost + kOutlierUnit - 1) / kOutlierUnit;
+      const int parts = want < 1 ? 1 : (want > kOutlierMaxParts ? kOutlierMaxParts : static_cast<int>(want));
+      const unsigned long long old =
+          atomicAdd(&sp->hdr.pack, (1ull << 32) | static_cast<unsigned long long>(parts));
+      const long long q = static_cast<long long>(old >> 32);
+      const long long first = static_cast<long long>(old & 0xffffffffull);
+      if (q < kOutlierCap && first + parts <= kOutlierPartCap) {
+        sp->entries[q] = OutlierEntry{f, b, static_cast<int>(first), parts};
+        for (int p = 0; p < parts; ++p) sp->partmap[first + p] = static_cast<int>(q);
+      }
+    }
+  }
+}
+
+// What the fused kernel reads when it starts: the number of outlier parts to run as tiles, 0 if
+// there are none or the list overflowed (then the teams sum every bag themselves).
+template <int MAXD>
+__device__ __forceinline__ int outlier_parts(const OutlierSpace<MAXD> *sp) {
+  const unsigned long long pack =
+      __hip_atomic_load(&sp->hdr.pack, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long entries = pack >> 32, parts = pack & 0xffffffffull;
+  return entries <= kOutlierCap && parts <= kOutlierPartCap ? static_cast<int>(parts) : 0;
+}
+
+// Called by every workgroup of the fused kernel when it has run out of tiles (by one thread):
+// the last one clears the header for the next launch.
+template <int MAXD> __device__ __forceinline__ void outliers_done(OutlierSpace<MAXD> *sp) {
+  const int done = __hip_atomic_fetch_add(&sp->hdr.finished, 1, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+  if (done == static_cast<int>(gridDim.x) - 1) {
+    const unsigned long long pack =
+        __hip_atomic_load(&sp->hdr.pack, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sp->hdr.last_entries = static_cast<int>(pack >> 32);
+    sp->hdr.last_parts = static_cast<int>(pack & 0xffffffffull);
+    __hip_atomic_store(&sp->hdr.finished, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&sp->hdr.pack, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+} // namespace rfx

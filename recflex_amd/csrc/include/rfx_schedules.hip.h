@@ -68,6 +68,12 @@ template <int BT> __device__ __forceinline__ int body_thread_id() {
 // indices fetched a round ahead, butterfly over the lookup lanes at the end.
 // No LDS and no barrier: only the wavefront that met the bag is involved.
 // ---------------------------------------------------------------------------------------------
+// a bag of more lookups than this is an outlier for a team with U lookups in flight on each of
+// Y lookup lanes: more than sixteen dependent rounds (at least 64 lookups)
+__host__ __device__ constexpr int long_bag_threshold(int u, int y) {
+  return 16 * u * y > 64 ? 16 * u * y : 64;
+}
+
 __host__ __device__ constexpr int pow2_at_least(int n) {
   int p = 1;
   while (p < n) p <<= 1;
@@ -171,7 +177,8 @@ __device__ __forceinline__ void
 team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
           const int *__restrict__ indices,
           const int *__restrict__ offsets, float *__restrict__ out, const int esum,
-          const int col_off, const int bag_begin, const int bag_end) {
+          const int col_off, const int bag_begin, const int bag_end,
+          const int skip_longer_than = 0x7fffffff) {
   using R = Row<DT, D>;
   constexpr int T = X * Y;
   static_assert(T >= 1 && T <= 64 && (T & (T - 1)) == 0, "team must be a power of two <= 64");
@@ -209,13 +216,16 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
     }
     // bags far longer than this schedule suits: the whole wavefront sums them, one at a time;
     // their teams then see an empty bag and leave the output alone
+    // (bags of more than skip_longer_than lookups were found ahead of the kernel and are summed
+    // by several workgroups as tiles of their own, rfx::find_outliers; nobody touches them here)
     int done_mask = 0;
+    constexpr int kLong = long_bag_threshold(U, Y);
     if constexpr (T < 64) {
-      constexpr int kLong = 16 * U * Y > 64 ? 16 * U * Y : 64;
 #pragma unroll
       for (int i = 0; i < UB; ++i) {
+        const bool skip = end[i] - beg[i] > skip_longer_than;
         const bool is_long = end[i] - beg[i] > kLong;
-        unsigned long long pending = __builtin_amdgcn_ballot_w64(is_long && lt == 0);
+        unsigned long long pending = __builtin_amdgcn_ballot_w64(is_long && !skip && lt == 0);
         while (pending) {                         // the same in every lane of the wavefront
           const int src = __builtin_ctzll(pending);
           pending &= pending - 1;
@@ -229,6 +239,13 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
           end[i] = beg[i];
         }
       }
+    } else {
+#pragma unroll
+      for (int i = 0; i < UB; ++i)
+        if (end[i] - beg[i] > skip_longer_than) {
+          done_mask |= 1 << i;
+          end[i] = beg[i];
+        }
     }
     int len_max = 0;
 #pragma unroll
@@ -596,19 +613,16 @@ __host__ __device__ constexpr int64_t split_region_floats(int d) {
   return static_cast<int64_t>(kSplitMaxTiles) * (d + 1);
 }
 
+// Part `part` of `parts` of bag `bag`: slot p of the bag is slots + p * slot_stride (D values),
+// counter its arrival counter.
 template <int BT, int DT, int D, int X, int U, int CHUNK>
 __device__ __forceinline__ void
-split_bags(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ table,
+split_part(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ table,
            const int *__restrict__ indices, const int *__restrict__ offsets,
-           float *__restrict__ out, const int esum, const int col_off, const int bag_begin,
-           const int bag_end, const int part, const int parts, float *__restrict__ region) {
-  if (parts <= 1) {
-    block_bags<BT, DT, D, X, U, CHUNK>(s, table, indices, offsets, out, esum, col_off, bag_begin,
-                                       bag_end);
-    return;
-  }
+           float *__restrict__ out, const int esum, const int col_off, const int bag,
+           const int part, const int parts, unsigned int *__restrict__ slots,
+           const int slot_stride, int *__restrict__ counter) {
   const int tid = body_thread_id<BT>();
-  const int bag = bag_begin;
   const int beg = offsets[bag];
   const int end = offsets[bag + 1];
   const int per = (end - beg + parts - 1) / parts;
@@ -624,12 +638,10 @@ split_bags(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ tab
   // when the memory counter has drained, so waiting for it before the arrival is announced
   // orders the slots before the counter; the finishing workgroup loads the slots only after its
   // arrival has returned.
-  unsigned int *slots = reinterpret_cast<unsigned int *>(region) +
-                        static_cast<int64_t>(bag) * parts * D;
-  int *counter = reinterpret_cast<int *>(region + static_cast<int64_t>(kSplitMaxTiles) * D) + bag;
   for (int j = tid; j < D; j += BT)
-    __hip_atomic_store(slots + part * D + j, __float_as_uint(block_column(s, j)),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(slots + static_cast<int64_t>(part) * slot_stride + j,
+                       __float_as_uint(block_column(s, j)), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (tid == 0) {
@@ -642,11 +654,30 @@ split_bags(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ tab
   for (int j = tid; j < D; j += BT) {
     float t = 0.f;
     for (int p = 0; p < parts; ++p)
-      t += __uint_as_float(__hip_atomic_load(slots + p * D + j, __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT));
+      t += __uint_as_float(__hip_atomic_load(slots + static_cast<int64_t>(p) * slot_stride + j,
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
     store_streaming(dst + j, t);
   }
   if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int BT, int DT, int D, int X, int U, int CHUNK>
+__device__ __forceinline__ void
+split_bags(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ table,
+           const int *__restrict__ indices, const int *__restrict__ offsets,
+           float *__restrict__ out, const int esum, const int col_off, const int bag_begin,
+           const int bag_end, const int part, const int parts, float *__restrict__ region) {
+  if (parts <= 1) {
+    block_bags<BT, DT, D, X, U, CHUNK>(s, table, indices, offsets, out, esum, col_off, bag_begin,
+                                       bag_end);
+    return;
+  }
+  const int bag = bag_begin;
+  unsigned int *slots = reinterpret_cast<unsigned int *>(region) +
+                        static_cast<int64_t>(bag) * parts * D;
+  int *counter = reinterpret_cast<int *>(region + static_cast<int64_t>(kSplitMaxTiles) * D) + bag;
+  split_part<BT, DT, D, X, U, CHUNK>(s, table, indices, offsets, out, esum, col_off, bag, part,
+                                     parts, slots, D, counter);
 }
 
 } // namespace rfx

@@ -26,7 +26,8 @@ class RecomInfo(ctypes.Structure):
         ("static_binding", ctypes.c_int32),
         ("num_candidates", ctypes.c_int32),
         ("xcd_segments", ctypes.c_int32),
-        ("reserved", ctypes.c_int32 * 5),
+        ("outliers", ctypes.c_int32),
+        ("reserved", ctypes.c_int32 * 4),
     ]
 
 

@@ -16,6 +16,8 @@ its library is missing.  Names:
 ``edge``           dims that force 8- and 4-byte row vectors and unaligned output columns
 ``longbags``       a dozen samples with bags of thousands of lookups (and some short and empty
                    ones) under the split-bag schedule: several workgroups per bag
+``c3s_outliers``   c3s with integer-valued tables, emitted with ``outliers=True``: bags beyond a
+                   schedule's threshold are found ahead of the kernel and run as tiles of their own
 ``fewbags``        8 fp32 features x 16 samples x 20 000 lookups, default schedules (split-bag);
                    ``fewbags_unsplit``: the same with one workgroup per bag, for comparison
 ``wide``           1 500 small features (several binding rounds per thread)
@@ -86,6 +88,8 @@ def _tuned(wl: Workload, fname: str) -> ModelSpec:
         kwargs.update(xcd_aware=True, xcd_segments=doc["xcd_segments"])
     else:
         kwargs.update(xcd_aware=False)      # the tuned walk is the flat one
+    if isinstance(doc, dict) and doc.get("outliers"):
+        kwargs["outliers"] = True
     return ModelSpec(wl, fs, occupancy, kwargs)
 
 
@@ -201,6 +205,8 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c3s": lambda: _default(make_workload("C3", batch=192, max_rows=60_000)),
     "c4s": lambda: _default(make_workload("C4", batch=128, num_features=48, max_rows=30_000)),
     "c5s": lambda: _default(make_workload("C5", batch=256, num_features=24, max_rows=50_000)),
+    "c3s_outliers": lambda: _default(make_workload("C3", batch=192, max_rows=60_000)._replace(
+        name="c3s_outliers", table_values="integer"), outliers=True),
     "variants": _variants,
     "edge": _edge,
     "longbags": _long_bags,

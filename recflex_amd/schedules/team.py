@@ -111,8 +111,13 @@ class TeamScheduleBase(ScheduleBase):
                  {p.items_per_thread}, {p.bags_per_team}, {p.vectors_per_pass}, {v.out_vec}>(
       {v.stage},
       {v.embed_table}, {v.indices}, {v.offsets}, {v.output},
-      {v.out_row_stride}, {v.embed_dim_offset}, {v.bag_begin}, {v.bag_end});
+      {v.out_row_stride}, {v.embed_dim_offset}, {v.bag_begin}, {v.bag_end}, {v.skip_long});
 '''
+
+    def LongBagThreshold(self, params: NamedTuple) -> int:
+        """rfx::long_bag_threshold(U, Y): more than sixteen dependent rounds of the team."""
+        p = self.team_params(params)
+        return max(64, 16 * p.items_per_thread * p.lanes_y)
 
     def EmitShmemType(self, params: NamedTuple) -> str:
         return "char"

@@ -71,6 +71,9 @@ class TuneConfig(NamedTuple):
     # run measurement workers in this process instead of one spawned process per measurement
     in_process: bool = True
     tile_bytes: int = DEFAULT_TILE_BYTES
+    # emit optimal/ with outlier tiles: bags far beyond their schedule's reach are found by a pass
+    # over the offsets ahead of the fused kernel and summed by several workgroups (skewed data)
+    outliers: bool = False
     # local-stage interference: "model" = every candidate of every feature is compiled into one
     # kernel of the whole model and timed while all other features run beside it;
     # "replicate" = per feature, the candidates side by side over the same data, replicated
@@ -221,14 +224,15 @@ class Tuner:
     def emit_codes(self, output_dir: str, feat_schedules: List[Tuple[ScheduleBase, NamedTuple]],
                    occupancy: int, inline: bool = True, timing: bool = False, tune: bool = False,
                    fixed_task_block_nums: List[int] = None, debug: bool = False,
-                   tile_bytes: int = None, host: bool = True, xcd_segments: int = 0) -> None:
+                   tile_bytes: int = None, host: bool = True, xcd_segments: int = 0,
+                   outliers: bool = False) -> None:
         os.makedirs(output_dir, exist_ok=True)
         emitter = CodeEmitter(feat_schedules)
         if host:
             emitter.emit_host(f"{output_dir}/preprocess.cpp", fixed_task_block_nums=fixed_task_block_nums)
         emitter.emit(f"{output_dir}/process.hip", occupancy=occupancy, timing=timing, inline=inline, tune=tune,
                      fixed_task_block_nums=fixed_task_block_nums, tile_bytes=tile_bytes,
-                     xcd_aware=xcd_segments > 0, xcd_segments=max(xcd_segments, 1))
+                     xcd_aware=xcd_segments > 0, xcd_segments=max(xcd_segments, 1), outliers=outliers)
         emitter.emit_cmake_list(f"{output_dir}/CMakeLists.txt", code_fname="process.hip",
                                 host_fname="preprocess.cpp" if host else None,
                                 subdirs=self.basic.subdirs, includes=self.basic.includes, links=self.basic.links,
@@ -555,16 +559,16 @@ class Tuner:
                           for a, b in zip(mix, opt_sched_params))
             opt_sched_params = mix
             print(f"occupancy: {opt_occupancy} (after the build climb), t(ns): {t}", flush=True)
-        if climbed or tile_bytes != tune_config.tile_bytes or xcd_segments:
+        if climbed or tile_bytes != tune_config.tile_bytes or xcd_segments or tune_config.outliers:
             # make the winning launch parameters the defaults of the optimal library
             self.emit_codes(output_dir=optimal, feat_schedules=opt_sched_params, occupancy=opt_occupancy,
                             inline=tune_config.inline, debug=tune_config.debug, tile_bytes=tile_bytes,
-                            xcd_segments=max(xcd_segments, 0))
+                            xcd_segments=max(xcd_segments, 0), outliers=tune_config.outliers)
             shutil.rmtree(f"{optimal}/build", ignore_errors=True)   # the copied CMake cache names another dir
             compile_build(f"{optimal}/build")
         with open(f"{optimal}/schedule.json", "w") as f:
             json.dump({"occupancy": opt_occupancy, "tile_bytes": tile_bytes,
-                       "xcd_segments": max(xcd_segments, 0),
+                       "xcd_segments": max(xcd_segments, 0), "outliers": tune_config.outliers,
                        "schedules": CodeEmitter(opt_sched_params).serialize_config()}, f, indent=1)
         return opt_occupancy, opt_sched_params
 

@@ -211,10 +211,32 @@ def test_split_bag_schedules_get_workspace_regions():
     regions, total = em.split_regions()
     assert regions == [-1, 0, -1, 2048 * 65] and total == 2048 * (65 + 129)
     src = em.emit_kernel(occupancy=4)
-    assert f"WORKSPACE_BYTES = {total * 4}LL" in src and "c_split_region[feat_idx]" in src
+    assert f"SPLIT_BYTES = {total * 4}LL" in src and "c_split_region[feat_idx]" in src
     assert "rfx::split_bags<" in src and "bind_tiles<NUM_FEATS, BLOCK_THREADS, HAS_SPLIT>" in src
     m = re.search(r"c_cand_gran\[\] = \{\s*([-\d,\s]+)\}", src)
     gran = [int(v) for v in m.group(1).split(",")]
     assert gran[1] == -1 and gran[3] == -1 and gran[0] > 0 and gran[2] > 0
     plain = CodeEmitter(fs[:1]).emit_kernel(occupancy=4)
-    assert "WORKSPACE_BYTES = 0LL" in plain and "c_split_region" not in plain
+    assert "SPLIT_BYTES = 0LL" in plain and "c_split_region" not in plain
+
+
+def test_outlier_tiles_are_emitted_on_request():
+    """outliers=True: a kernel that lists the bags beyond each feature's threshold (its
+    schedule's reach, and at least 128 KiB of traffic), one block-wide body per (element type,
+    dim), the list and its partial sums in the workspace.  Nothing of it otherwise."""
+    fs = [default_schedule(MetaData(32), 4), default_schedule(MetaData(128), 1),
+          default_schedule(MetaData(32), 30), default_schedule(MetaData(64, "half"), 900)]
+    em = CodeEmitter(fs)
+    thr, keys, body_of = em.long_bag_tables()
+    # 132-byte lookups: 993 lookups make 128 KiB; 516-byte lookups: 255; the split-bag feature
+    # takes bags of any length itself
+    assert thr == [993, 255, 993, 0] and keys == [(0, 32), (0, 128)] and body_of == [0, 1, 0, -1]
+    assert all(t >= s.LongBagThreshold(p) for t, (s, p) in zip(thr[:3], fs[:3]))
+    src = em.emit_kernel(occupancy=4, outliers=True)
+    assert "#define RFX_OUTLIERS 1" in src and "OutlierKnl" in src and "MAX_LONG_DIM = 128" in src
+    assert src.count("rfx::split_part<") == 2 and "rfx::outliers_done(d_outliers)" in src
+    assert "c_long_thr[feat_idx]" in src
+    plain = em.emit_kernel(occupancy=4)
+    assert "#define RFX_OUTLIERS 0" in plain and "OutlierKnl" not in plain and "c_long_thr" not in plain
+    with pytest.raises(AssertionError):
+        em.emit_kernel(occupancy=4, outliers=True, timing=True)

@@ -1,0 +1,76 @@
+"""GPU parity of a library emitted with outlier tiles (bags found ahead of the kernel and summed
+by several workgroups)."""
+
+import numpy as np
+import pytest
+
+from helpers import oracle_output, require_lib
+
+pytestmark = pytest.mark.gpu
+
+
+def _inject(rng, wl, indices, offsets, plan):
+    """plan: {feature: [extra lookups, ...]} -- each entry lengthens one random bag."""
+    indices, offsets = list(indices), list(offsets)
+    for f, extras in plan.items():
+        lens = np.diff(offsets[f]).astype(np.int64)
+        for extra in extras:
+            lens[rng.integers(0, wl.batch)] += extra
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        indices[f] = rng.integers(0, wl.features[f].rows, int(off[-1])).astype(np.int32)
+        offsets[f] = off
+    return indices, offsets
+
+
+@pytest.mark.parametrize("case", ["none", "few", "many", "overflow"])
+def test_outlier_tiles_are_bit_exact(case):
+    """No outlier at all; a few bags of 300 to 20 000 lookups in features of every kind of
+    schedule; some hundred outliers; more than the list holds (512), where the launch falls back
+    to a wavefront per outlier.  Three launches each on one workspace, whose list header and
+    arrival counters must be back at zero afterwards.  Integer-valued tables: bit for bit."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    wl = prebuilt.model_spec("c3s_outliers").workload
+    assert wl.table_values == "integer"
+    dev = torch.device("cuda", 0)
+    print(f"[case] c3s_outliers {case}: F={wl.num_features} B={wl.batch}", flush=True)
+    tables = gen_tables(wl, dev)
+    host_tables = [t.cpu().numpy() for t in tables]
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib("c3s_outliers"))
+    assert layer.workspace is not None
+    rng = np.random.default_rng(len(case))
+    base_idx, base_off = gen_inputs(wl)
+    for launch in range(3):
+        feats = rng.permutation(wl.num_features)
+        if case == "none":
+            plan = {}
+        elif case == "few":
+            plan = {int(f): [int(x)] for f, x in zip(feats[:6], (300, 2000, 20000, 4200, 5000, 9000))}
+        elif case == "many":
+            plan = {int(f): [2000 + 371 * k for k in range(12)] for f in feats[:10]}
+        else:
+            plan = {int(f): [4000] * (4 * wl.batch) for f in feats[:4]}
+        indices, offsets = _inject(rng, wl, base_idx, base_off, plan)
+        d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+        d_off = [torch.from_numpy(o).to(dev) for o in offsets]
+        got = layer.forward_indices(d_idx, d_off).cpu().numpy()
+        want = oracle_output(wl, host_tables, indices, offsets)
+        bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+        assert bad.size == 0, f"launch {launch}: {len(bad)} elements differ, first at {bad[:5].tolist()}"
+        ws = layer.workspace.cpu().numpy()
+        # the outlier space follows the split regions (none here): header (32 ints), 512 entries
+        # of 4 ints, 512 counters
+        assert not ws[:3].any(), f"launch {launch}: list header not cleared: {ws[:3].tolist()}"
+        # what the launch found: entries beyond its schedule's threshold and 128 KiB of traffic
+        thr = [max(s.LongBagThreshold(p), -(-131072 // (4 * f.dim + 4)))
+               for (s, p), f in zip(prebuilt.model_spec("c3s_outliers").feat_schedules, wl.features)]
+        expect = sum(int((np.diff(o) > t).sum()) for o, t in zip(offsets, thr))
+        assert int(ws[3]) == expect, (int(ws[3]), expect)
+        if case == "overflow":
+            assert expect > 512
+        elif case != "none":
+            assert 0 < expect <= 512 and int(ws[4]) >= 2 * expect
+        assert not ws[32 + 2048:32 + 2048 + 512].any(), f"launch {launch}: arrival counters not reset"
