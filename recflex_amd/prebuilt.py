@@ -17,7 +17,8 @@ its library is missing.  Names:
 ``longbags``       a dozen samples with bags of thousands of lookups (and some short and empty
                    ones) under the split-bag schedule: several workgroups per bag
 ``c3s_outliers``   c3s with integer-valued tables, emitted with ``outliers=True``: bags beyond a
-                   schedule's threshold are found ahead of the kernel and run as tiles of their own
+                   schedule's threshold are found ahead of the kernel and run as tiles of their
+                   own; every tenth feature under the split-bag schedule
 ``fewbags``        8 fp32 features x 16 samples x 20 000 lookups, default schedules (split-bag);
                    ``fewbags_unsplit``: the same with one workgroup per bag, for comparison
 ``wide``           1 500 small features (several binding rounds per thread)
@@ -160,6 +161,19 @@ def _long_bags() -> ModelSpec:
     return ModelSpec(wl, scheds, DEFAULT_OCCUPANCY)
 
 
+def _c3s_outliers() -> ModelSpec:
+    """c3s with integer-valued tables and outlier tiles; every tenth feature runs the split-bag
+    schedule, so that the library's workspace holds split regions and the outlier list."""
+    wl = make_workload("C3", batch=192, max_rows=60_000)._replace(name="c3s_outliers",
+                                                                   table_values="integer")
+    spec = _default(wl, outliers=True)
+    fs = list(spec.feat_schedules)
+    for f in range(0, len(fs), 10):
+        sched = SplitBagSchedule(fs[f][0].meta, BLOCK_THREADS)
+        fs[f] = (sched, sched.GenParamCandidates()[0])
+    return spec._replace(feat_schedules=fs)
+
+
 def _few_bags(split: bool) -> ModelSpec:
     """Fewer bags than the device has workgroups, each of 20 000 lookups."""
     feats = tuple(FeatureSpec(2_000_000, d, "float", 20000.0, False, 0.0, 1.0)
@@ -205,8 +219,7 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c3s": lambda: _default(make_workload("C3", batch=192, max_rows=60_000)),
     "c4s": lambda: _default(make_workload("C4", batch=128, num_features=48, max_rows=30_000)),
     "c5s": lambda: _default(make_workload("C5", batch=256, num_features=24, max_rows=50_000)),
-    "c3s_outliers": lambda: _default(make_workload("C3", batch=192, max_rows=60_000)._replace(
-        name="c3s_outliers", table_values="integer"), outliers=True),
+    "c3s_outliers": _c3s_outliers,
     "variants": _variants,
     "edge": _edge,
     "longbags": _long_bags,

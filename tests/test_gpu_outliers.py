@@ -33,8 +33,10 @@ def test_outlier_tiles_are_bit_exact(case):
     from recflex_amd.rec_modules import FeatEmbed
     from recflex_amd.workloads import gen_inputs, gen_tables
 
-    wl = prebuilt.model_spec("c3s_outliers").workload
+    spec = prebuilt.model_spec("c3s_outliers")
+    wl = spec.workload
     assert wl.table_values == "integer"
+    assert sum(type(s).__name__ == "SplitBagSchedule" for s, _ in spec.feat_schedules) == 10
     dev = torch.device("cuda", 0)
     print(f"[case] c3s_outliers {case}: F={wl.num_features} B={wl.batch}", flush=True)
     tables = gen_tables(wl, dev)
@@ -52,7 +54,7 @@ def test_outlier_tiles_are_bit_exact(case):
         elif case == "many":
             plan = {int(f): [2000 + 371 * k for k in range(12)] for f in feats[:10]}
         else:
-            plan = {int(f): [4000] * (4 * wl.batch) for f in feats[:4]}
+            plan = {int(f): [4000] * (4 * wl.batch) for f in feats[:8]}
         indices, offsets = _inject(rng, wl, base_idx, base_off, plan)
         d_idx = [torch.from_numpy(i).to(dev) for i in indices]
         d_off = [torch.from_numpy(o).to(dev) for o in offsets]
@@ -60,14 +62,19 @@ def test_outlier_tiles_are_bit_exact(case):
         want = oracle_output(wl, host_tables, indices, offsets)
         bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
         assert bad.size == 0, f"launch {launch}: {len(bad)} elements differ, first at {bad[:5].tolist()}"
+        # the outlier space follows the split regions of every tenth feature: header (32 ints),
+        # 512 entries of 4 ints, 512 counters, 4096 part -> entry, 4096 slots of 128 floats
         ws = layer.workspace.cpu().numpy()
-        # the outlier space follows the split regions (none here): header (32 ints), 512 entries
-        # of 4 ints, 512 counters
+        ws = ws[len(ws) - (32 + 2048 + 512 + 4096 + 4096 * 128):]
         assert not ws[:3].any(), f"launch {launch}: list header not cleared: {ws[:3].tolist()}"
-        # what the launch found: entries beyond its schedule's threshold and 128 KiB of traffic
-        thr = [max(s.LongBagThreshold(p), -(-131072 // (4 * f.dim + 4)))
-               for (s, p), f in zip(prebuilt.model_spec("c3s_outliers").feat_schedules, wl.features)]
-        expect = sum(int((np.diff(o) > t).sum()) for o, t in zip(offsets, thr))
+        assert not ws[32 + 2048:32 + 2048 + 512].any(), f"launch {launch}: arrival counters not reset"
+        # what the launch found: bags beyond their schedule's threshold and 128 KiB of traffic
+        # (split-bag features take bags of any length themselves)
+        expect = 0
+        for (sched, params), feat, off in zip(spec.feat_schedules, wl.features, offsets):
+            if sched.LongBagThreshold(params) > 0:
+                thr = max(sched.LongBagThreshold(params), -(-131072 // (4 * feat.dim + 4)))
+                expect += int((np.diff(off) > thr).sum())
         assert int(ws[3]) == expect, (int(ws[3]), expect)
         if case == "overflow":
             assert expect > 512

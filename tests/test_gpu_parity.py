@@ -329,7 +329,7 @@ def test_every_schedule_variant_on_ragged_batches(batch, seed):
     assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
 
 
-@pytest.mark.parametrize("name", ["c3s", "wider", "longbags"])
+@pytest.mark.parametrize("name", ["c3s", "wider", "longbags", "c3s_outliers"])
 def test_launch_replays_inside_a_hip_graph(name):
     """recom_process is a single kernel launch on the caller's stream (binding happens on the
     device, no host-side task mapping, no copies), so a serving loop can capture it once and
