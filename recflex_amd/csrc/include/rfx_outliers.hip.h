@@ -21,8 +21,8 @@
 
 namespace rfx {
 
-constexpr int kOutlierCap = 512;             // entries
-constexpr int kOutlierPartCap = 4096;        // parts of all entries together
+constexpr int kOutlierCap = 4096;            // entries
+constexpr int kOutlierPartCap = 16384;       // parts of all entries together
 constexpr int kOutlierUnit = 128 * 1024;     // traffic of one part
 constexpr int kOutlierMaxParts = 64;
 

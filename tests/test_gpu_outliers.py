@@ -8,12 +8,18 @@ from helpers import oracle_output, require_lib
 
 pytestmark = pytest.mark.gpu
 
+CAP, PARTS = 4096, 16384      # rfx::kOutlierCap, rfx::kOutlierPartCap
+
 
 def _inject(rng, wl, indices, offsets, plan):
-    """plan: {feature: [extra lookups, ...]} -- each entry lengthens one random bag."""
+    """plan: {feature: [extra lookups, ...]} -- each entry lengthens one random bag; an int
+    instead of a list lengthens every bag of the feature."""
     indices, offsets = list(indices), list(offsets)
     for f, extras in plan.items():
         lens = np.diff(offsets[f]).astype(np.int64)
+        if isinstance(extras, int):
+            lens += extras
+            extras = []
         for extra in extras:
             lens[rng.integers(0, wl.batch)] += extra
         off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
@@ -25,7 +31,7 @@ def _inject(rng, wl, indices, offsets, plan):
 @pytest.mark.parametrize("case", ["none", "few", "many", "overflow"])
 def test_outlier_tiles_are_bit_exact(case):
     """No outlier at all; a few bags of 300 to 20 000 lookups in features of every kind of
-    schedule; some hundred outliers; more than the list holds (512), where the launch falls back
+    schedule; some hundred outliers; more than the list holds (4 096), where the launch falls back
     to a wavefront per outlier.  Three launches each on one workspace, whose list header and
     arrival counters must be back at zero afterwards.  Integer-valued tables: bit for bit."""
     import torch
@@ -54,7 +60,7 @@ def test_outlier_tiles_are_bit_exact(case):
         elif case == "many":
             plan = {int(f): [2000 + 371 * k for k in range(12)] for f in feats[:10]}
         else:
-            plan = {int(f): [4000] * (4 * wl.batch) for f in feats[:8]}
+            plan = {int(f): 2500 for f in feats[:60]}
         indices, offsets = _inject(rng, wl, base_idx, base_off, plan)
         d_idx = [torch.from_numpy(i).to(dev) for i in indices]
         d_off = [torch.from_numpy(o).to(dev) for o in offsets]
@@ -63,11 +69,11 @@ def test_outlier_tiles_are_bit_exact(case):
         bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
         assert bad.size == 0, f"launch {launch}: {len(bad)} elements differ, first at {bad[:5].tolist()}"
         # the outlier space follows the split regions of every tenth feature: header (32 ints),
-        # 512 entries of 4 ints, 512 counters, 4096 part -> entry, 4096 slots of 128 floats
+        # CAP entries of 4 ints, CAP counters, PARTS part -> entry, PARTS slots of 128 floats
         ws = layer.workspace.cpu().numpy()
-        ws = ws[len(ws) - (32 + 2048 + 512 + 4096 + 4096 * 128):]
+        ws = ws[len(ws) - (32 + 4 * CAP + CAP + PARTS + PARTS * 128):]
         assert not ws[:3].any(), f"launch {launch}: list header not cleared: {ws[:3].tolist()}"
-        assert not ws[32 + 2048:32 + 2048 + 512].any(), f"launch {launch}: arrival counters not reset"
+        assert not ws[32 + 4 * CAP:32 + 5 * CAP].any(), f"launch {launch}: arrival counters not reset"
         # what the launch found: bags beyond their schedule's threshold and 128 KiB of traffic
         # (split-bag features take bags of any length themselves)
         expect = 0
@@ -77,7 +83,6 @@ def test_outlier_tiles_are_bit_exact(case):
                 expect += int((np.diff(off) > thr).sum())
         assert int(ws[3]) == expect, (int(ws[3]), expect)
         if case == "overflow":
-            assert expect > 512
+            assert expect > CAP
         elif case != "none":
-            assert 0 < expect <= 512 and int(ws[4]) >= 2 * expect
-        assert not ws[32 + 2048:32 + 2048 + 512].any(), f"launch {launch}: arrival counters not reset"
+            assert 0 < expect <= CAP and int(ws[4]) >= 2 * expect
