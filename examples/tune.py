@@ -74,10 +74,11 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--xcd_segments_candidates", type=str,
                         help="comma-separated tile-walk settings swept in the global stage "
                              "(-1 = flat, n > 0 = n segments per XCD)")
-    parser.add_argument("--outliers", action="store_true",
+    parser.add_argument("--outliers", choices=["auto", "on", "off"], default="auto",
                         help="emit the optimal library with outlier tiles: bags far longer than "
                              "their feature's schedule suits are found ahead of the fused kernel "
-                             "and summed by several workgroups (for data with skewed bag lengths)")
+                             "and summed by several workgroups (for data with skewed bag lengths); "
+                             "auto = on if the sampled batches hold such a bag")
     parser.add_argument("--build_climb_trials", type=int, default=0,
                         help="global stage: that many single-feature variants of the winning mix are "
                              "built as production kernels and timed; the faster ones are adopted")
@@ -155,7 +156,7 @@ def create_tune_config(args: argparse.Namespace) -> TuneConfig:
     kwargs = {"register_census": not args.no_register_census,
               "build_climb_trials": args.build_climb_trials,
               "build_climb_top_k": args.build_climb_top_k,
-              "climb_passes": args.climb_passes, "outliers": args.outliers}
+              "climb_passes": args.climb_passes, "outliers": {"auto": None, "on": True, "off": False}[args.outliers]}
     if args.tile_bytes:
         kwargs["tile_bytes"] = args.tile_bytes
     if args.xcd_segments_candidates:

@@ -72,8 +72,9 @@ class TuneConfig(NamedTuple):
     in_process: bool = True
     tile_bytes: int = DEFAULT_TILE_BYTES
     # emit optimal/ with outlier tiles: bags far beyond their schedule's reach are found by a pass
-    # over the offsets ahead of the fused kernel and summed by several workgroups (skewed data)
-    outliers: bool = False
+    # over the offsets ahead of the fused kernel and summed by several workgroups (skewed data).
+    # None: decided from the sampled batches -- on if any of them holds such a bag
+    outliers: Optional[bool] = None
     # local-stage interference: "model" = every candidate of every feature is compiled into one
     # kernel of the whole model and timed while all other features run beside it;
     # "replicate" = per feature, the candidates side by side over the same data, replicated
@@ -541,6 +542,18 @@ class Tuner:
                 occu_opt_sched_params[i].append(self.feat_sched_param_candidates[feat_id][opt_idx])
         return occu_opt_sched_params
 
+    def has_outlier_bags(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]]) -> bool:
+        """True if a sampled batch holds a bag that a library with outlier tiles would run as
+        tiles of its own (beyond its feature's schedule and at least a tile's traffic)."""
+        thresholds, _, _ = CodeEmitter(sched_params).long_bag_tables()
+        batches = getattr(self, "batches", None)
+        if not batches:
+            return False
+        for thr, feat in zip(thresholds, batches):
+            if thr > 0 and any(len(off) > 1 and int(np.diff(off).max()) > thr for _, off in feat):
+                return True
+        return False
+
     def solve(self, measured_times: Dict[int, Dict[int, List[float]]],
               tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
         occu_opt_sched_params = self.select_per_occupancy(measured_times, tune_config.occupancies)
@@ -559,16 +572,20 @@ class Tuner:
                           for a, b in zip(mix, opt_sched_params))
             opt_sched_params = mix
             print(f"occupancy: {opt_occupancy} (after the build climb), t(ns): {t}", flush=True)
-        if climbed or tile_bytes != tune_config.tile_bytes or xcd_segments or tune_config.outliers:
+        outliers = tune_config.outliers
+        if outliers is None:
+            outliers = self.has_outlier_bags(opt_sched_params)
+            print(f"outlier tiles: {'on' if outliers else 'off'} (decided from the sampled batches)", flush=True)
+        if climbed or tile_bytes != tune_config.tile_bytes or xcd_segments or outliers:
             # make the winning launch parameters the defaults of the optimal library
             self.emit_codes(output_dir=optimal, feat_schedules=opt_sched_params, occupancy=opt_occupancy,
                             inline=tune_config.inline, debug=tune_config.debug, tile_bytes=tile_bytes,
-                            xcd_segments=max(xcd_segments, 0), outliers=tune_config.outliers)
+                            xcd_segments=max(xcd_segments, 0), outliers=outliers)
             shutil.rmtree(f"{optimal}/build", ignore_errors=True)   # the copied CMake cache names another dir
             compile_build(f"{optimal}/build")
         with open(f"{optimal}/schedule.json", "w") as f:
             json.dump({"occupancy": opt_occupancy, "tile_bytes": tile_bytes,
-                       "xcd_segments": max(xcd_segments, 0), "outliers": tune_config.outliers,
+                       "xcd_segments": max(xcd_segments, 0), "outliers": bool(outliers),
                        "schedules": CodeEmitter(opt_sched_params).serialize_config()}, f, indent=1)
         return opt_occupancy, opt_sched_params
 

@@ -306,3 +306,24 @@ def test_automatic_tile_size_rule():
     assert auto_tile_bytes([off(8192, 300)] * 400, [516] * 400, [516] * 400, 1024) == 256 * 1024
     # a grid of one workgroup and an empty batch do not divide by zero
     assert auto_tile_bytes([np.zeros(1, dtype=np.int64)], [36], [36], 0) == 64 * 1024
+
+
+def test_outlier_tiles_are_switched_on_by_the_sampled_data():
+    """tune.py --outliers auto: the optimal library gets outlier tiles if a sampled batch holds
+    a bag beyond its feature's schedule that carries at least 128 KiB of traffic."""
+    from recflex_amd.code_emitter import MetaData
+    from recflex_amd.schedules import default_schedule
+    from recflex_amd.tuning.tuner import Tuner
+    fs = [default_schedule(MetaData(32), 4), default_schedule(MetaData(128), 1)]
+    # 132-byte lookups: 993 of them make 128 KiB; 516-byte lookups: 255
+    tuner = Tuner.__new__(Tuner)
+    short = np.array([0, 3, 3, 900], dtype=np.int32)
+    tuner.batches = [[(None, short)], [(None, np.array([0, 1, 2, 250], dtype=np.int32))]]
+    assert not tuner.has_outlier_bags(fs)
+    tuner.batches = [[(None, short), (None, np.array([0, 5, 1200, 1201], dtype=np.int32))],
+                     [(None, np.array([0, 1, 2, 3], dtype=np.int32))]]
+    assert tuner.has_outlier_bags(fs)
+    tuner.batches = [[(None, short)], [(None, np.array([0, 1, 300, 301], dtype=np.int32))]]
+    assert tuner.has_outlier_bags(fs)
+    del tuner.batches
+    assert not tuner.has_outlier_bags(fs)
