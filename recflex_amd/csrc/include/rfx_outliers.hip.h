@@ -6,7 +6,8 @@
 // emitted with outliers=True launches find_outliers ahead of the fused kernel: it walks all
 // offsets of the batch, and every bag longer than its schedule's threshold
 // (rfx::long_bag_threshold) becomes an entry {feature, bag, first part, parts} of a list in the
-// caller's workspace, parts = its traffic / kOutlierUnit (1..kOutlierMaxParts).  The fused
+// caller's workspace, parts = its traffic / kOutlierUnit (1..kOutlierMaxParts; 128, 256 and
+// 512 KiB per part give 227, 219 and 234 us on a 100-feature model with lognormal bag lengths).  The fused
 // kernel runs the parts of all entries as its first tiles, each like a part of a split bag
 // (rfx::split_part: partial sums in a slot, arrival counter, the last one adds the slots in
 // part order and writes the output), and its teams leave those bags alone.  If the list
@@ -23,7 +24,7 @@ namespace rfx {
 
 constexpr int kOutlierCap = 4096;            // entries
 constexpr int kOutlierPartCap = 16384;       // parts of all entries together
-constexpr int kOutlierUnit = 128 * 1024;     // traffic of one part
+constexpr int kOutlierUnit = 256 * 1024;     // traffic of one part
 constexpr int kOutlierMaxParts = 64;
 
 struct OutlierHeader {

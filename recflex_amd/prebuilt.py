@@ -19,6 +19,9 @@ its library is missing.  Names:
 ``c3s_outliers``   c3s with integer-valued tables, emitted with ``outliers=True``: bags beyond a
                    schedule's threshold are found ahead of the kernel and run as tiles of their
                    own; every tenth feature under the split-bag schedule
+``c3_skew``        C3 with bag lengths from a lognormal (sigma 1.5) of the same means and
+                   integer-valued tables, default schedules, emitted with outlier tiles;
+                   ``c3_skew_plain``: the same without them
 ``fewbags``        8 fp32 features x 16 samples x 20 000 lookups, default schedules (split-bag);
                    ``fewbags_unsplit``: the same with one workgroup per bag, for comparison
 ``wide``           1 500 small features (several binding rounds per thread)
@@ -174,6 +177,14 @@ def _c3s_outliers() -> ModelSpec:
     return spec._replace(feat_schedules=fs)
 
 
+def _c3_skew(outliers: bool) -> ModelSpec:
+    """Heavy-tailed bag lengths: some thousand bags per batch far beyond their schedule."""
+    wl = make_workload("C3")
+    wl = wl._replace(name="c3_skew", table_values="integer",
+                     features=tuple(f._replace(len_sigma=1.5) for f in wl.features))
+    return _default(wl, outliers=outliers)
+
+
 def _few_bags(split: bool) -> ModelSpec:
     """Fewer bags than the device has workgroups, each of 20 000 lookups."""
     feats = tuple(FeatureSpec(2_000_000, d, "float", 20000.0, False, 0.0, 1.0)
@@ -223,6 +234,8 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "variants": _variants,
     "edge": _edge,
     "longbags": _long_bags,
+    "c3_skew": lambda: _c3_skew(True),
+    "c3_skew_plain": lambda: _c3_skew(False),
     "fewbags": lambda: _few_bags(True),
     "fewbags_unsplit": lambda: _few_bags(False),
     "wide": _wide,

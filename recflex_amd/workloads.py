@@ -41,6 +41,9 @@ class FeatureSpec(NamedTuple):
     fixed_len: bool     # every bag has exactly round(mean_bag) lookups
     empty_frac: float   # share of bags forced to length 0
     zipf_alpha: float   # 0 = uniform indices
+    # > 0: bag lengths from a lognormal of mean mean_bag and this sigma of the logarithm instead
+    # of a Poisson (a heavy tail: at 1.5 the longest of 2 048 bags is some hundred means long)
+    len_sigma: float = 0.0
 
 
 class Workload(NamedTuple):
@@ -165,6 +168,9 @@ def gen_feature_inputs(spec: FeatureSpec, batch: int, seed_seq: np.random.SeedSe
     rng = np.random.Generator(np.random.PCG64(seed_seq))
     if spec.fixed_len:
         lens = np.full(batch, int(round(spec.mean_bag)), dtype=np.int64)
+    elif spec.len_sigma > 0:
+        mu = np.log(max(spec.mean_bag, 0.05)) - spec.len_sigma ** 2 / 2
+        lens = np.floor(rng.lognormal(mu, spec.len_sigma, batch) + rng.random(batch)).astype(np.int64)
     else:
         lens = rng.poisson(spec.mean_bag, batch).astype(np.int64)
     if spec.empty_frac > 0:
