@@ -90,8 +90,9 @@ int recom_get_max_concurrent_blocks(int32_t *out);
 /* Bytes of recom_process_args.d_workspace this library needs: 0 unless a feature runs a
  * schedule that splits bags over workgroups, then 2048 * (D_f + 1) * 4 bytes for each such
  * feature (rounded up to 128); a library with outlier tiles adds its list of outliers and
- * their partial sums (147 584 + 65 536 * max dim bytes).  Replaces the extra-buffer sizes the
- * reference's host preprocessors report per batch (RecFlex/code_emitter/codegen.py:149-160,
+ * their partial sums (entries * (36 + 16 * max dim) + 128 bytes; 4 096 entries up to 128
+ * features, 16 384 beyond).  Replaces the extra-buffer sizes the reference's host
+ * preprocessors report per batch (RecFlex/code_emitter/codegen.py:149-160,
  * extra_buffer_offsets). */
 int recom_get_workspace_bytes(int64_t *out);
 

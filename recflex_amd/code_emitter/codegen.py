@@ -44,6 +44,11 @@ BIND_ONCE_MIN_FEATS = 2048
 OUTLIER_MIN_BYTES = 128 * 1024
 
 
+def outlier_capacity(num_feats: int) -> int:
+    """Entries of the outlier list of a library emitted with outlier tiles (four parts each)."""
+    return 4096 if num_feats <= 128 else 16384
+
+
 def _c_array(ctype: str, name: str, values: List[int], per_line: int = 16) -> str:
     lines = []
     for i in range(0, len(values), per_line):
@@ -226,7 +231,7 @@ constexpr bool HAS_SPLIT = SPLIT_BYTES > 0;
 #define RFX_OUTLIERS {1 if outliers else 0}
 constexpr bool OUTLIERS = RFX_OUTLIERS;
 constexpr int MAX_LONG_DIM = {max_long_dim};
-using OutlierSpace = rfx::OutlierSpace<MAX_LONG_DIM>;
+using OutlierSpace = rfx::OutlierSpace<MAX_LONG_DIM, {outlier_capacity(num_feats)}>;
 constexpr long long WORKSPACE_BYTES = SPLIT_BYTES + (OUTLIERS ? (long long)sizeof(OutlierSpace) : 0LL);
 static_assert(rfx::kBindMaxSplitTiles == {SPLIT_MAX_TILES} && rfx::kSplitGran == {SPLIT_GRANULARITY},
               "workspace regions were sized for this");
@@ -372,7 +377,7 @@ extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
     const int64_t *__restrict__ d_arg_buffer_offsets, const int batch,
     OutlierSpace *__restrict__ d_outliers) {
   const rfx::IoView io{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch};
-  rfx::find_outliers<NUM_FEATS, MAX_LONG_DIM>(d_outliers, io, c_long_thr, c_lookup_bytes);
+  rfx::find_outliers<NUM_FEATS>(d_outliers, io, c_long_thr, c_lookup_bytes);
 }
 ''' if outliers else ''
         outlier_begin = '''

@@ -11,7 +11,7 @@
 // kernel runs the parts of all entries as its first tiles, each like a part of a split bag
 // (rfx::split_part: partial sums in a slot, arrival counter, the last one adds the slots in
 // part order and writes the output), and its teams leave those bags alone.  If the list
-// overflows (more than kOutlierCap bags or kOutlierPartCap parts) the launch falls back to the
+// overflows (more than CAP bags or 4 * CAP parts) the launch falls back to the
 // wavefront path for all of them.  The workgroup that finishes last puts the list header back
 // to zero for the next launch.
 //
@@ -22,8 +22,8 @@
 
 namespace rfx {
 
-constexpr int kOutlierCap = 4096;            // entries
-constexpr int kOutlierPartCap = 16384;       // parts of all entries together
+// The list holds CAP entries and 4 * CAP parts; the emitter sizes it by the model (4 096 entries
+// up to 128 features, 16 384 beyond).
 constexpr int kOutlierUnit = 256 * 1024;     // traffic of one part
 constexpr int kOutlierMaxParts = 64;
 
@@ -38,18 +38,20 @@ struct OutlierEntry {
 };
 
 // MAXD: largest embedding dimension among the features that can have outliers, rounded up to 4
-template <int MAXD> struct OutlierSpace {
+template <int MAXD, int CAP> struct OutlierSpace {
+  static constexpr int kCap = CAP;           // entries
+  static constexpr int kPartCap = 4 * CAP;   // parts of all entries together
   OutlierHeader hdr;
-  OutlierEntry entries[kOutlierCap];
-  int counters[kOutlierCap];                 // arrival counters, zero between launches
-  int partmap[kOutlierPartCap];              // part -> entry
-  unsigned int slots[kOutlierPartCap][MAXD]; // partial sums
+  OutlierEntry entries[kCap];
+  int counters[kCap];                        // arrival counters, zero between launches
+  int partmap[kPartCap];                     // part -> entry
+  unsigned int slots[kPartCap][MAXD];        // partial sums
 };
 
 // One thread per (feature, bag); grid (x: bags, y: features), any size.
-template <int F, int MAXD>
+template <int F, typename Space>
 __device__ __forceinline__ void
-find_outliers(OutlierSpace<MAXD> *__restrict__ sp, const IoView &io,
+find_outliers(Space *__restrict__ sp, const IoView &io,
               const int *__restrict__ long_thr, const int *__restrict__ lookup_bytes) {
   for (int f = blockIdx.y; f < F; f += gridDim.y) {
     const int thr = long_thr[f];
@@ -65,7 +67,7 @@ find_outliers(OutlierSpace<MAXD> *__restrict__ sp, const IoView &io,
           atomicAdd(&sp->hdr.pack, (1ull << 32) | static_cast<unsigned long long>(parts));
       const long long q = static_cast<long long>(old >> 32);
       const long long first = static_cast<long long>(old & 0xffffffffull);
-      if (q < kOutlierCap && first + parts <= kOutlierPartCap) {
+      if (q < Space::kCap && first + parts <= Space::kPartCap) {
         sp->entries[q] = OutlierEntry{f, b, static_cast<int>(first), parts};
         for (int p = 0; p < parts; ++p) sp->partmap[first + p] = static_cast<int>(q);
       }
@@ -75,17 +77,17 @@ find_outliers(OutlierSpace<MAXD> *__restrict__ sp, const IoView &io,
 
 // What the fused kernel reads when it starts: the number of outlier parts to run as tiles, 0 if
 // there are none or the list overflowed (then the teams sum every bag themselves).
-template <int MAXD>
-__device__ __forceinline__ int outlier_parts(const OutlierSpace<MAXD> *sp) {
+template <typename Space>
+__device__ __forceinline__ int outlier_parts(const Space *sp) {
   const unsigned long long pack =
       __hip_atomic_load(&sp->hdr.pack, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const unsigned long long entries = pack >> 32, parts = pack & 0xffffffffull;
-  return entries <= kOutlierCap && parts <= kOutlierPartCap ? static_cast<int>(parts) : 0;
+  return entries <= Space::kCap && parts <= Space::kPartCap ? static_cast<int>(parts) : 0;
 }
 
 // Called by every workgroup of the fused kernel when it has run out of tiles (by one thread):
 // the last one clears the header for the next launch.
-template <int MAXD> __device__ __forceinline__ void outliers_done(OutlierSpace<MAXD> *sp) {
+template <typename Space> __device__ __forceinline__ void outliers_done(Space *sp) {
   const int done = __hip_atomic_fetch_add(&sp->hdr.finished, 1, __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
   if (done == static_cast<int>(gridDim.x) - 1) {
