@@ -629,6 +629,11 @@ split_part(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ tab
   const int pbeg = min(end, beg + part * per);
   const int pend = min(end, pbeg + per);
   block_sum_range<BT, DT, D, X, U, CHUNK>(s, table, indices, pbeg, pend, tid);
+  if (parts == 1) {                 // the whole bag: nothing to combine
+    float *dst = out + static_cast<int64_t>(bag) * esum + col_off;
+    for (int j = tid; j < D; j += BT) store_streaming(dst + j, block_column(s, j));
+    return;
+  }
 
   // Partial sums and counters are read and written with device-scope atomic loads and stores:
   // the workgroups of one bag run on different XCDs, whose L2 caches do not see each other's
