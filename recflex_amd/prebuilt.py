@@ -24,6 +24,8 @@ its library is missing.  Names:
                    ``c3_skew_plain``: the same without them
 ``fewbags``        8 fp32 features x 16 samples x 20 000 lookups, default schedules (split-bag);
                    ``fewbags_unsplit``: the same with one workgroup per bag, for comparison
+``manysplit``      17 fp16 features of dim 256 under the split-bag schedule: 36 MB of workspace,
+                   more than the static array of ``recom_process_static_workspace`` may hold
 ``wide``           1 500 small features (several binding rounds per thread)
 ``wider``          2 500 small features (bound once per launch by the binding kernel)
 """
@@ -199,6 +201,15 @@ def _few_bags(split: bool) -> ModelSpec:
     return ModelSpec(wl, fs, 8)
 
 
+def _many_split() -> ModelSpec:
+    """More split-bag workspace than a library's static device array may hold (32 MiB)."""
+    feats = tuple(FeatureSpec(5000 + f, 256, "half", 3000.0, False, 0.0, 1.0) for f in range(17))
+    wl = Workload("manysplit", 8, 1717, feats, "integer")
+    sched = SplitBagSchedule(MetaData(256, "half"), BLOCK_THREADS)
+    params = sched.GenParamCandidates()[0]
+    return ModelSpec(wl, [(sched, params)] * len(feats), DEFAULT_OCCUPANCY)
+
+
 def _wide(num_features: int = 1500, name: str = "wide") -> ModelSpec:
     """Many small features: several rounds of the binding loop per thread and a prefix array
     longer than a wavefront scan covers at once, as in the reference's own models.  Above
@@ -238,6 +249,7 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c3_skew_plain": lambda: _c3_skew(False),
     "fewbags": lambda: _few_bags(True),
     "fewbags_unsplit": lambda: _few_bags(False),
+    "manysplit": _many_split,
     "wide": _wide,
     "wider": lambda: _wide(2500, "wider"),
     "b128": lambda: _other_block_size(128),
@@ -313,9 +325,23 @@ def fixture_tune_config(**overrides):
     return TuneConfig(**kwargs)
 
 
+# the ablation modes of the fixture: tiles of 2 KiB, so that its small features still get several
+# tiles each and a frozen binding differs from one tile per feature
+ABLATION_TILE_BYTES = 2048
+ABLATION_OCCUPANCY = 4
+ABLATION_MUTATED_FEATURE = 0
+
+
+def fixture_default_mix(tuner) -> list:
+    """The default schedule of every feature, as entries of the tuner's candidate lists."""
+    return [tuner.feat_sched_param_candidates[f][k] for f, k in enumerate(tuner.default_choices()[0])]
+
+
 def build_tune_fixture(model_dir: str) -> str:
-    """Local-stage kernels of the fixture model plus ``default/`` (default schedules, with the
-    generated host front end), all under ``_models/tune_fixture``."""
+    """Local-stage kernels of the fixture model, ``default/`` (default schedules, with the
+    generated host front end) and the kernels of the tuner's ablation modes (one per candidate
+    of ``tune_naive``, the mutations of one feature, the two frozen bindings), all under
+    ``_models/tune_fixture``: a GPU machine then only measures."""
     import multiprocessing as mp
     if mp.get_start_method(allow_none=True) != "spawn":
         mp.set_start_method("spawn", force=True)
@@ -325,4 +351,10 @@ def build_tune_fixture(model_dir: str) -> str:
     mean_lens = [float(np.mean([len(i) / max(1, len(o) - 1) for i, o in feat])) for feat in tuner.batches]
     fs = default_feat_schedules(tuner.metas, mean_lens, BLOCK_THREADS)
     build_model(os.path.join(tune_fixture_dir(), "default"), fs, rebuild=True, occupancy=None)
+    ablation = fixture_tune_config(recompile=True, tile_bytes=ABLATION_TILE_BYTES)
+    tuner.compile_naive(ablation)
+    mix = fixture_default_mix(tuner)
+    tuner.compile_mutation(mix, ABLATION_OCCUPANCY, ABLATION_MUTATED_FEATURE, ablation)
+    for choice in ("mean", "max"):
+        tuner.compile_fixed_thread_binding(mix, choice, ablation._replace(remeasure=True))
     return tune_fixture_dir()

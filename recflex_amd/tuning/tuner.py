@@ -183,7 +183,17 @@ class Tuner:
                 for params in schedule.GenParamCandidates():
                     self.feat_sched_param_candidates[feat_id].append([schedule, params])
             if not self.feat_sched_param_candidates[feat_id]:
-                raise ValueError(f"feature {feat_id}: its schedule classes produced no candidate")
+                # e.g. a template whose parameter space has no member for rows this wide: tune
+                # nothing for this feature, run the default schedule
+                from recflex_amd.schedules import default_schedule
+                lens = [len(i) / max(1, len(o) - 1) for i, o in self.batches[feat_id]]
+                sched, params = default_schedule(self.metas[feat_id], float(np.mean(lens)) if lens else 1.0,
+                                                 self.basic.block_threads)
+                print(f"feature {feat_id}: its schedule classes "
+                      f"({', '.join(type(s).__name__ for s in self.feat_schedules[feat_id])}) have no "
+                      f"candidate for dim {self.metas[feat_id].embed_dim} {self.metas[feat_id].data_type}; "
+                      f"using the default schedule {type(sched).__name__}{tuple(params)}", flush=True)
+                self.feat_sched_param_candidates[feat_id].append([sched, params])
 
     def write_data_files(self):
         """Per-feature ``data/f{i}.npz`` under ``codegen_dir`` (what the workers read) and, for
@@ -826,10 +836,11 @@ class Tuner:
 
     # ------------------------------------------------------------------ validation / ablations
 
-    def mutation_validation(self, opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]], opt_occupancy: int,
-                            mut_feat_id: int, tune_config: TuneConfig) -> Tuple[List[float], int]:
-        """Whole-kernel time with feature ``mut_feat_id`` switched to each of its candidates in
-        turn; returns the times and the index of the tuner's own pick."""
+    def compile_mutation(self, opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]], opt_occupancy: int,
+                         mut_feat_id: int, tune_config: TuneConfig) -> int:
+        """Emit and build ``mutation_f{id}/m{k}``: the whole model with feature ``mut_feat_id``
+        switched to its candidate ``k``, for every ``k`` (no GPU needed).  Returns the index of
+        the candidate ``opt_sched_params`` holds for that feature (-1 if it is not in the list)."""
         mutation_dir = f"{self.basic.codegen_dir}/mutation_f{mut_feat_id}"
         candidates = self.feat_sched_param_candidates[mut_feat_id]
         opt_idx = -1
@@ -845,6 +856,15 @@ class Tuner:
             if self._build_full(output_dir, mut_sched_params, opt_occupancy, tune_config):
                 jobs.append((output_dir, f"{output_dir}/build"))
         self._schedule_builds(jobs, tune_config)
+        return opt_idx
+
+    def mutation_validation(self, opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]], opt_occupancy: int,
+                            mut_feat_id: int, tune_config: TuneConfig) -> Tuple[List[float], int]:
+        """Whole-kernel time with feature ``mut_feat_id`` switched to each of its candidates in
+        turn; returns the times and the index of the tuner's own pick."""
+        mutation_dir = f"{self.basic.codegen_dir}/mutation_f{mut_feat_id}"
+        candidates = self.feat_sched_param_candidates[mut_feat_id]
+        opt_idx = self.compile_mutation(opt_sched_params, opt_occupancy, mut_feat_id, tune_config)
 
         manager = self._measure_manager(tune_config)
         for candidate_id in range(len(candidates)):
@@ -855,13 +875,14 @@ class Tuner:
                  for candidate_id in range(len(candidates))]
         return times, opt_idx
 
-    def tune_naive(self, tune_config: TuneConfig) -> Tuple[List[Tuple[ScheduleBase, NamedTuple]], float]:
-        """Every candidate of every feature measured alone on the GPU (no interference, no
-        occupancy control); the per-feature winners are fused and the whole kernel timed."""
-        def get_output_build_dir(feat_id: int, sched_param_id: int):
-            output_dir = f"{self.basic.codegen_dir}/naive/f{feat_id}/s{sched_param_id}"
-            return output_dir, f"{output_dir}/build"
+    def _naive_dirs(self, feat_id: int, sched_param_id: int) -> Tuple[str, str]:
+        output_dir = f"{self.basic.codegen_dir}/naive/f{feat_id}/s{sched_param_id}"
+        return output_dir, f"{output_dir}/build"
 
+    def compile_naive(self, tune_config: TuneConfig) -> None:
+        """Emit and build ``naive/f{feat}/s{k}``: one single-feature kernel per candidate (no GPU
+        needed; features with the same candidate list share their builds)."""
+        get_output_build_dir = self._naive_dirs
         jobs = []
         for feat_id in range(self.num_feats):
             for sched_param_id, sched_param in enumerate(self.feat_sched_param_candidates[feat_id]):
@@ -873,6 +894,12 @@ class Tuner:
                                     debug=tune_config.debug, tile_bytes=tune_config.tile_bytes, host=False)
                     jobs.append((output_dir, build_dir))
         self._schedule_builds(jobs, tune_config)
+
+    def tune_naive(self, tune_config: TuneConfig) -> Tuple[List[Tuple[ScheduleBase, NamedTuple]], float]:
+        """Every candidate of every feature measured alone on the GPU (no interference, no
+        occupancy control); the per-feature winners are fused and the whole kernel timed."""
+        get_output_build_dir = self._naive_dirs
+        self.compile_naive(tune_config)
 
         manager = None if tune_config.in_process else TaskManager(tune_config.gpu_ids)
         for feat_id in range(self.num_feats):
@@ -904,10 +931,11 @@ class Tuner:
             manager.join()
         return opt_sched_params, self._read_kernel_time(output_dir, tune_config)
 
-    def tune_fixed_thread_binding(self, opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]], choice: str,
-                                  tune_config: TuneConfig) -> Tuple[List[int], float]:
-        """Ablation: the number of tiles per feature is frozen to the mean / max over the sampled
-        batches of what the run-time binding chose, and baked into the kernel."""
+    def compile_fixed_thread_binding(self, opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]],
+                                     choice: str, tune_config: TuneConfig) -> List[int]:
+        """Write ``fixed_thread_binding_{choice}/task_blocks.txt`` (the tiles per feature the
+        run-time binding would choose for each sampled batch, computed on the CPU), freeze their
+        mean / max into a kernel and build it (no GPU needed).  Returns the frozen counts."""
         assert choice in ["max", "mean"]
         output_dir = f"{self.basic.codegen_dir}/fixed_thread_binding_{choice}"
         fixed_blocks_path = f"{output_dir}/task_blocks.txt"
@@ -935,6 +963,14 @@ class Tuner:
         if self._build_full(output_dir, opt_sched_params, None, tune_config,
                             fixed_task_block_nums=fixed_task_blocks):
             self._schedule_builds([(output_dir, f"{output_dir}/build")], tune_config)
+        return fixed_task_blocks
+
+    def tune_fixed_thread_binding(self, opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]], choice: str,
+                                  tune_config: TuneConfig) -> Tuple[List[int], float]:
+        """Ablation: the number of tiles per feature is frozen to the mean / max over the sampled
+        batches of what the run-time binding chose, and baked into the kernel."""
+        fixed_task_blocks = self.compile_fixed_thread_binding(opt_sched_params, choice, tune_config)
+        output_dir = f"{self.basic.codegen_dir}/fixed_thread_binding_{choice}"
         manager = self._measure_manager(tune_config)
         self._kernel_time(output_dir, tune_config, manager)
         if manager:
