@@ -264,3 +264,39 @@ def algorithmic_bytes(wl: Workload, num_lookups: Sequence[int]) -> int:
         total += int(L) * (row_bytes(spec.dim, spec.data_type) + 4)
         total += (wl.batch + 1) * 4 + wl.batch * spec.dim * 4
     return total
+
+
+CACHE_LINE = 128       # bytes fetched from HBM at a time on an MI355X
+
+
+def distinct_row_lines(indices: np.ndarray, stride: int, payload: int, line: int = CACHE_LINE) -> int:
+    """Distinct ``line``-byte memory lines that hold the payload bytes of the rows ``indices``
+    of a table whose rows are ``stride`` bytes apart (table base aligned to a line): narrow rows
+    share lines, wide rows span several."""
+    if len(indices) == 0:
+        return 0
+    rows = np.unique(np.asarray(indices, dtype=np.int64))
+    first = rows * stride // line
+    last = (rows * stride + payload - 1) // line
+    # rows are sorted, so their line intervals are too: a row can only share its first line(s)
+    # with the row before it
+    prev_last = np.concatenate([[-1], last[:-1]])
+    return int(np.maximum(last - np.maximum(first, prev_last + 1) + 1, 0).sum())
+
+
+def compulsory_bytes(wl: Workload, indices: Sequence[np.ndarray], offsets: Sequence[np.ndarray],
+                     line: int = CACHE_LINE) -> int:
+    """Bytes that must cross the HBM pins for one batch even with perfect caches: every distinct
+    memory line of the table rows the batch touches once, plus the index arrays, the offset
+    arrays and the pooled output (each rounded up to whole lines).  Always at most
+    ``algorithmic_bytes``, which counts a row as often as it is looked up."""
+    def lines(nbytes: int) -> int:
+        return -(-nbytes // line)
+    total = 0
+    for spec, idx, off in zip(wl.features, indices, offsets):
+        used = idx[:int(off[-1])]
+        total += distinct_row_lines(used, row_stride(spec.dim, spec.data_type),
+                                    row_bytes(spec.dim, spec.data_type), line) * line
+        total += lines(len(used) * 4) * line + lines(len(off) * 4) * line
+    total += lines(wl.batch * wl.embed_dim_sum * 4) * line
+    return total

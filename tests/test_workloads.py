@@ -74,3 +74,34 @@ def test_algorithmic_bytes_formula():
     wl2 = make_workload("C2")
     idx, _ = gen_inputs(wl2)
     assert algorithmic_bytes(wl2, [len(i) for i in idx]) == 26 * (4096 * 260 + 4097 * 4 + 4096 * 256)
+
+
+def test_compulsory_bytes_counts_each_memory_line_once():
+    """Against a brute-force set of touched line numbers, for rows narrower than a line (several
+    rows per line), rows of whole lines, and the 144-byte int8 rows that straddle lines."""
+    from recflex_amd.workloads import (FeatureSpec, Workload, algorithmic_bytes, compulsory_bytes,
+                                       distinct_row_lines, row_bytes, row_stride)
+    rng = np.random.default_rng(5)
+    for dim, dt in ((8, "float"), (32, "float"), (128, "float"), (16, "half"), (128, "int8"), (24, "int8")):
+        stride, payload = row_stride(dim, dt), row_bytes(dim, dt)
+        idx = rng.integers(0, 500, 3000)
+        want = set()
+        for r in idx.tolist():
+            want.update(range(r * stride // 128, (r * stride + payload - 1) // 128 + 1))
+        assert distinct_row_lines(idx, stride, payload) == len(want), (dim, dt)
+    assert distinct_row_lines(np.zeros(0, np.int32), 64, 64) == 0
+    # one row looked up a thousand times is one row's lines
+    assert distinct_row_lines(np.full(1000, 7), 512, 512) == 4
+    feats = (FeatureSpec(1000, 32, "float", 3.0, False, 0.0, 1.05), FeatureSpec(50, 128, "int8", 9.0, False, 0.1, 0.0))
+    wl = Workload("t", 64, 3, feats)
+    indices, offsets = gen_inputs(wl)
+    comp = compulsory_bytes(wl, indices, offsets)
+    alg = algorithmic_bytes(wl, [len(i) for i in indices])
+    out_lines = -(-64 * 160 * 4 // 128)
+    expect = out_lines * 128
+    for spec, i, o in zip(feats, indices, offsets):
+        expect += distinct_row_lines(i, row_stride(spec.dim, spec.data_type), row_bytes(spec.dim, spec.data_type)) * 128
+        expect += -(-len(i) * 4 // 128) * 128 + -(-len(o) * 4 // 128) * 128
+    assert comp == expect and comp % 128 == 0
+    # hot rows are counted once: far fewer bytes than the algorithmic count for the 50-row table
+    assert comp < alg + 4 * 128
