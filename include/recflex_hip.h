@@ -61,7 +61,8 @@ typedef struct recom_info {
   int32_t reserved[4];
 } recom_info;
 
-#define RECOM_ABI_VERSION 3     /* 3: recom_get_workspace_bytes, d_workspace / workspace_bytes */
+#define RECOM_ABI_VERSION 4     /* 4: the once-per-launch binding table of very wide models moved
+                                 * into the workspace */
 
 /* Static description of the emitted kernel.  No reference counterpart as a function: the
  * reference bakes the same numbers into process.cu (EMBED_DIM_SUM, block_threads,
@@ -91,9 +92,10 @@ int recom_get_max_concurrent_blocks(int32_t *out);
  * schedule that splits bags over workgroups, then 2048 * (D_f + 1) * 4 bytes for each such
  * feature (rounded up to 128); a library with outlier tiles adds its list of outliers and
  * their partial sums (entries * (36 + 16 * max dim) + 128 bytes; 4 096 entries up to 128
- * features, 16 384 beyond).  Replaces the extra-buffer sizes the reference's host
- * preprocessors report per batch (RecFlex/code_emitter/codegen.py:149-160,
- * extra_buffer_offsets). */
+ * features, 16 384 beyond); a library of more than 2048 features adds the table into which a
+ * one-workgroup kernel binds the model once per launch (12 bytes per feature).  Replaces the
+ * extra-buffer sizes the reference's host preprocessors report per batch
+ * (RecFlex/code_emitter/codegen.py:149-160, extra_buffer_offsets). */
 int recom_get_workspace_bytes(int64_t *out);
 
 typedef struct recom_launch_info {
@@ -157,7 +159,8 @@ typedef struct recom_process_args {
    * (the kernel then stores 16 bytes at a time), and d_output aligned likewise. */
   int64_t output_row_stride;
   /* Workspace of the schedules that give one bag to several workgroups (batches of few, very
-   * long bags): device memory of at least recom_get_workspace_bytes() bytes, 16-byte aligned,
+   * long bags), of the outlier tiles and of the once-per-launch binding of very wide models:
+   * device memory of at least recom_get_workspace_bytes() bytes, 16-byte aligned,
    * caller allocated.  It must be all zero before the first launch that uses it; every launch
    * leaves its arrival counters at zero again, so it is cleared once, not per launch.  Launches
    * that may overlap (different streams) need a workspace each.  Ignored (may be NULL) by a
@@ -175,9 +178,7 @@ typedef struct recom_process_args {
  * Never allocates.  A library emitted with outlier tiles (recom_info.outliers) launches a small
  * kernel ahead that walks the offsets and lists the outlier bags in the workspace.
  * A library of more than 2048 features launches a one-workgroup kernel ahead
- * of the fused one that binds the model for this batch into a static device array of the
- * library; the array has one slot per stream (eight), launches on one stream share theirs, and
- * a ninth stream on the same device is refused with hipErrorOutOfMemory (2). */
+ * of the fused one that binds the model for this batch into a table in the workspace. */
 int recom_process(const recom_process_args *args);
 
 /* ------------------------------------------------------------------------------------------

@@ -224,15 +224,20 @@ constexpr bool TIMING = {"true" if timing else "false"};
 constexpr bool STATIC_BINDING = {"true" if fixed_task_block_nums else "false"};
 #define RFX_BIND_ONCE {1 if bind_once else 0}
 constexpr bool BIND_ONCE = RFX_BIND_ONCE;
-// bytes of caller workspace the split-bag schedules need (0: no schedule splits bags)
+// bytes of workspace the split-bag schedules need (0: no schedule splits bags)
 constexpr long long SPLIT_BYTES = {workspace_floats * 4}LL;
+#define RFX_HAS_SPLIT {1 if workspace_floats > 0 else 0}
 constexpr bool HAS_SPLIT = SPLIT_BYTES > 0;
 // outlier bags found ahead of the kernel and run as tiles of their own (rfx_outliers.hip.h)
 #define RFX_OUTLIERS {1 if outliers else 0}
 constexpr bool OUTLIERS = RFX_OUTLIERS;
 constexpr int MAX_LONG_DIM = {max_long_dim};
 using OutlierSpace = rfx::OutlierSpace<MAX_LONG_DIM, {outlier_capacity(num_feats)}>;
-constexpr long long WORKSPACE_BYTES = SPLIT_BYTES + (OUTLIERS ? (long long)sizeof(OutlierSpace) : 0LL);
+constexpr long long OUTLIER_BYTES = OUTLIERS ? (long long)sizeof(OutlierSpace) : 0LL;
+// the binding table of a model that is bound once per launch (rfx::bind_once) comes last
+constexpr long long BOUND_OFFSET = (SPLIT_BYTES + OUTLIER_BYTES + 255) / 256 * 256;
+constexpr long long BOUND_BYTES = BIND_ONCE ? (long long)sizeof(rfx::BoundTables<NUM_FEATS>) : 0LL;
+constexpr long long WORKSPACE_BYTES = BIND_ONCE ? BOUND_OFFSET + BOUND_BYTES : SPLIT_BYTES + OUTLIER_BYTES;
 static_assert(rfx::kBindMaxSplitTiles == {SPLIT_MAX_TILES} && rfx::kSplitGran == {SPLIT_GRANULARITY},
               "workspace regions were sized for this");
 
@@ -350,10 +355,6 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
                          f"      d_schedule_choice, {fixed_arg}, gridDim.x);\n  (void)d_bound;")
             bound_src = "s_bind."
         bind_kernel = f'''
-// the binding tables of the launches in flight, one slot per stream (rfx::bind_slot_for)
-static __device__ __align__(256) char
-    g_bound[BIND_ONCE ? rfx::kBindSlots * sizeof(rfx::BoundTables<NUM_FEATS>) : 256];
-
 // One workgroup binds the whole model for this launch (models of thousands of features).
 extern "C" __global__ void __launch_bounds__(1024) BindKnl(
     const int64_t *__restrict__ d_io_ptrs, const char *__restrict__ d_arg_buffers,
@@ -366,9 +367,7 @@ extern "C" __global__ void __launch_bounds__(1024) BindKnl(
                                   c_cand_begin, c_cand_gran, d_schedule_choice, {fixed_arg},
                                   grid_blocks);
 }}
-''' if bind_once else '''
-static __device__ __align__(256) char g_bound[256];     // unused: every workgroup binds for itself
-'''
+''' if bind_once else ''
 
         outlier_kernel = '''
 // Finds the bags that are too long for their feature's schedule (one thread per bag).
@@ -487,24 +486,10 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
 
     def emit_process_func(self, timing: bool = False, occupancy: int = None) -> str:
         return '''
-extern "C" int recom_process(const recom_process_args *a) {
-  if (!a || !a->d_embed_table_ptrs || !a->d_output || a->batch < 0 ||
-      (!a->d_io_ptrs && (!a->d_arg_buffers || !a->d_arg_buffer_offsets)))
-    return static_cast<int>(hipErrorInvalidValue);
-  if (!TIMING && a->d_times) return static_cast<int>(hipErrorInvalidValue);
-  if (a->tile_bytes < 0 || a->grid_blocks < 0 || a->xcd_segments > 4096)
-    return static_cast<int>(hipErrorInvalidValue);
-  // the output: dense rows unless a stride is given; aligned for the widest store of the kernel
+// Launches the kernels of one call on a->stream; `workspace` holds WORKSPACE_BYTES bytes (the
+// caller's buffer or the library's static array) or is null when the library needs none.
+static int launch_kernels(const recom_process_args *a, void *workspace) {
   const int64_t row_stride = a->output_row_stride ? a->output_row_stride : EMBED_DIM_SUM;
-  if (row_stride < EMBED_DIM_SUM || row_stride > 0x7fffffff || row_stride % OUT_VEC != 0 ||
-      reinterpret_cast<uintptr_t>(a->d_output) % (OUT_VEC * sizeof(float)) != 0)
-    return static_cast<int>(hipErrorInvalidValue);
-  // split-bag schedules keep partial sums and arrival counters in the caller's workspace
-  if (WORKSPACE_BYTES > 0 && (!a->d_workspace || a->workspace_bytes < WORKSPACE_BYTES ||
-                    reinterpret_cast<uintptr_t>(a->d_workspace) % 16 != 0))
-    return static_cast<int>(hipErrorInvalidValue);
-  if (a->batch == 0) return static_cast<int>(hipSuccess);
-
   const rfx::LaunchState *st = nullptr;
   hipError_t e = rfx::get_launch_state(FusedKnl, BLOCK_THREADS, OCCUPANCY, &st);
   if (e != hipSuccess) return static_cast<int>(e);
@@ -519,9 +504,8 @@ extern "C" int recom_process(const recom_process_args *a) {
   const char *arg_buffers = static_cast<const char *>(a->d_arg_buffers);
   int batch = a->batch, tile_arg = tile_bytes, xcd_arg = xcd_segments;
   int stride_arg = static_cast<int>(row_stride);
-  void *workspace = a->d_workspace;
-  void *outlier_space = OUTLIERS ? static_cast<char *>(a->d_workspace) + SPLIT_BYTES : nullptr;
-  void *bound = nullptr;
+  void *outlier_space = OUTLIERS ? static_cast<char *>(workspace) + SPLIT_BYTES : nullptr;
+  void *bound = BIND_ONCE ? static_cast<char *>(workspace) + BOUND_OFFSET : nullptr;
 #if RFX_OUTLIERS
   {
     void *outlier_args[] = {const_cast<int64_t **>(&a->d_io_ptrs), &arg_buffers,
@@ -534,13 +518,6 @@ extern "C" int recom_process(const recom_process_args *a) {
   }
 #endif
 #if RFX_BIND_ONCE
-  e = rfx::bind_slot_for(
-      [](char **p) {
-        return hipGetSymbolAddress(reinterpret_cast<void **>(p), HIP_SYMBOL(g_bound));
-      },
-      sizeof(rfx::BoundTables<NUM_FEATS>), a->stream, &bound);
-  if (e != hipSuccess) return static_cast<int>(e);
-  if (!bound) return static_cast<int>(hipErrorOutOfMemory);    // more streams than slots
   int grid_arg = grid;
   void *bind_args[] = {const_cast<int64_t **>(&a->d_io_ptrs), &arg_buffers,
                        const_cast<int64_t **>(&a->d_arg_buffer_offsets), &batch, &tile_arg,
@@ -559,6 +536,30 @@ extern "C" int recom_process(const recom_process_args *a) {
   e = hipLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
                       kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream));
   return static_cast<int>(e);
+}
+
+// checked before any HIP call
+static bool valid_process_args(const recom_process_args *a) {
+  if (!a || !a->d_embed_table_ptrs || !a->d_output || a->batch < 0 ||
+      (!a->d_io_ptrs && (!a->d_arg_buffers || !a->d_arg_buffer_offsets)))
+    return false;
+  if (!TIMING && a->d_times) return false;
+  if (a->tile_bytes < 0 || a->grid_blocks < 0 || a->xcd_segments > 4096) return false;
+  // the output: dense rows unless a stride is given; aligned for the widest store of the kernel
+  const int64_t row_stride = a->output_row_stride ? a->output_row_stride : EMBED_DIM_SUM;
+  return row_stride >= EMBED_DIM_SUM && row_stride <= 0x7fffffff && row_stride % OUT_VEC == 0 &&
+         reinterpret_cast<uintptr_t>(a->d_output) % (OUT_VEC * sizeof(float)) == 0;
+}
+
+extern "C" int recom_process(const recom_process_args *a) {
+  if (!valid_process_args(a)) return static_cast<int>(hipErrorInvalidValue);
+  // split-bag schedules, outlier tiles and the once-per-launch binding keep their partial sums,
+  // lists and tables in the caller's workspace
+  if (WORKSPACE_BYTES > 0 && (!a->d_workspace || a->workspace_bytes < WORKSPACE_BYTES ||
+                    reinterpret_cast<uintptr_t>(a->d_workspace) % 16 != 0))
+    return static_cast<int>(hipErrorInvalidValue);
+  if (a->batch == 0) return static_cast<int>(hipSuccess);
+  return launch_kernels(a, WORKSPACE_BYTES > 0 ? a->d_workspace : nullptr);
 }
 '''
 

@@ -121,47 +121,4 @@ inline hipError_t get_launch_state(K kernel, int block_threads, int want_occupan
   return hipSuccess;
 }
 
-// Slots of the binding table that a very wide model computes once per launch.  The table lives
-// in a file-scope device array of the generated library (nothing is allocated), cut into
-// kBindSlots slots.  Launches on one stream run in order and share a slot; a different stream
-// gets a different slot, which it keeps for the life of the process.  When every slot belongs to
-// another stream, `out` stays null and the caller reports an error: more than kBindSlots streams
-// launching one such library on one device are not supported.
-constexpr int kBindSlots = 8;
-
-struct BindSlots {
-  char *base = nullptr;                   // device address of the array on this device
-  const void *streams[kBindSlots] = {};
-  int used = 0;
-};
-
-// `resolve` yields the device address of the library's array on the current device
-// (hipGetSymbolAddress); it is called once per device.
-template <typename Resolve>
-inline hipError_t bind_slot_for(Resolve resolve, const size_t bytes_per_slot, const void *stream,
-                                void **out) {
-  static BindSlots slots[kMaxDevices];
-  static std::mutex mu;
-  *out = nullptr;
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
-  std::lock_guard<std::mutex> lock(mu);
-  BindSlots &s = slots[dev];
-  if (!s.base) {
-    e = resolve(&s.base);
-    if (e != hipSuccess) return e;
-  }
-  int slot = -1;
-  for (int i = 0; i < s.used; ++i)
-    if (s.streams[i] == stream) slot = i;
-  if (slot < 0 && s.used < kBindSlots) {
-    slot = s.used++;
-    s.streams[slot] = stream;
-  }
-  if (slot >= 0) *out = s.base + static_cast<size_t>(slot) * bytes_per_slot;
-  return hipSuccess;
-}
-
 } // namespace rfx

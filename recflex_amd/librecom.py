@@ -60,7 +60,7 @@ class RecomProcessArgs(ctypes.Structure):
     ]
 
 
-RECOM_ABI_VERSION = 3
+RECOM_ABI_VERSION = 4
 EXPORTED_SYMBOLS = ("recom_get_info", "recom_get_feature_tables", "recom_get_candidate_counts",
                     "recom_get_launch_info", "recom_get_workspace_bytes",
                     "recom_get_max_concurrent_blocks", "recom_process")
