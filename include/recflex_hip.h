@@ -107,6 +107,8 @@ typedef struct recom_launch_info {
   int32_t num_vgprs;          /* vector registers per lane */
   int32_t static_lds_bytes;
   int32_t lds_bytes_per_cu;
+  int32_t padded_api_occupancy; /* hipOccupancyMaxActiveBlocksPerMultiprocessor with the pad */
+  int32_t reserved[3];
 } recom_launch_info;
 
 /* How FusedKnl is launched on the current device: the pieces of the reference's
@@ -145,8 +147,10 @@ typedef struct recom_process_args {
   /* tuning builds: device int32[F], the candidate schedule each feature runs in this launch
    * (clamped to the feature's candidate count); NULL = candidate 0 everywhere */
   const int32_t *d_schedule_choice;
-  /* timing builds only: device uint64[F], the kernel ADDS each feature's workgroup-ticks
-   * (s_memtime) to it; caller zeroes it.  Replaces the per-block clock() array
+  /* timing builds only: device uint64[F + 2], the kernel ADDS each feature's workgroup-ticks
+   * (s_memtime) to entries 0..F-1, the ticks every workgroup spends before its first tile (the
+   * run-time binding) to entry F and every workgroup's ticks from start to end to entry F + 1;
+   * caller zeroes it.  Replaces the per-block clock() array
    * (RecFlex/code_emitter/codegen.py:301-316,388-401).  NULL runs a timing build untimed;
    * must be NULL for other builds. */
   unsigned long long *d_times;

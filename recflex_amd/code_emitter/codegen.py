@@ -320,14 +320,25 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
 ''' if timing else ''
         timing_init = f'''
   __shared__ unsigned int s_ticks[NUM_FEATS];
+  const unsigned long long t_kernel_begin = d_times ? __builtin_amdgcn_s_memtime() : 0;
   if (d_times)
     for (int f = threadIdx.x; f < NUM_FEATS; f += {vars_.BLOCK_THREADS}) s_ticks[f] = 0;
+''' if timing else ''
+        # ticks every workgroup spends before its first tile (the binding), entry NUM_FEATS
+        timing_bound = '''
+  const unsigned long long t_bound = d_times ? __builtin_amdgcn_s_memtime() : 0;
 ''' if timing else ''
         timing_flush = f'''
   if (d_times) {{
     __syncthreads();
     for (int f = threadIdx.x; f < NUM_FEATS; f += {vars_.BLOCK_THREADS})
       if (s_ticks[f]) atomicAdd(&d_times[f], static_cast<unsigned long long>(s_ticks[f]));
+    if (threadIdx.x == 0) {{
+      // beyond the per-feature entries: the workgroup's ticks before its first tile, and all of
+      // its ticks
+      atomicAdd(&d_times[NUM_FEATS], t_bound - t_kernel_begin);
+      atomicAdd(&d_times[NUM_FEATS + 1], __builtin_amdgcn_s_memtime() - t_kernel_begin);
+    }}
   }}
 ''' if timing else ''
 
@@ -425,7 +436,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
 {stage_decl}{timing_init}
   const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
 {bind_call}
-
+{timing_bound}
 {outlier_begin}
   // Tiles are ordered by feature.  Workgroup i runs on XCD i % XCDS.  With xcd_segments > 0 the
   // tile space is cut into XCDS * xcd_segments equal segments and segment s belongs to XCD
@@ -579,6 +590,7 @@ extern "C" int recom_get_launch_info(recom_launch_info *out) {
   out->num_vgprs = st->num_vgprs;
   out->static_lds_bytes = st->static_lds;
   out->lds_bytes_per_cu = st->lds_per_cu;
+  out->padded_api_occupancy = st->padded_api_occupancy;
   return static_cast<int>(hipSuccess);
 }
 

@@ -23,6 +23,7 @@ struct LaunchState {
   int num_vgprs = 0;      // vector registers per lane of the kernel
   int static_lds = 0;     // static LDS of the kernel (bytes)
   int lds_per_cu = 0;     // LDS of one compute unit (bytes)
+  int padded_api_occupancy = 0;  // the occupancy API's answer with the pad
 };
 
 // gfx950: 4 SIMDs per CU, 512 vector registers per lane and SIMD (allocated in blocks of 8),
@@ -97,6 +98,11 @@ inline hipError_t init_launch_state(K kernel, int block_threads, int want_occupa
     }
     st->occupancy = want_occupancy;
     st->dyn_lds = static_cast<int>(dyn);
+  }
+  st->padded_api_occupancy = occ_api;
+  if (st->dyn_lds > 0) {
+    e = occupancy_of(kernel, block_threads, static_cast<size_t>(st->dyn_lds), &st->padded_api_occupancy);
+    if (e != hipSuccess) return e;
   }
   st->ready = true;
   return hipSuccess;

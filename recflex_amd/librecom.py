@@ -34,10 +34,11 @@ class RecomInfo(ctypes.Structure):
 class RecomLaunchInfo(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in (
         "compute_units", "occupancy", "dyn_lds_bytes", "natural_occupancy", "api_occupancy",
-        "num_vgprs", "static_lds_bytes", "lds_bytes_per_cu")]
+        "num_vgprs", "static_lds_bytes", "lds_bytes_per_cu", "padded_api_occupancy")] + \
+        [("reserved", ctypes.c_int32 * 3)]
 
     def as_dict(self):
-        return {n: getattr(self, n) for n, _ in self._fields_}
+        return {n: getattr(self, n) for n, _ in self._fields_ if n != "reserved"}
 
 
 class RecomProcessArgs(ctypes.Structure):

@@ -131,6 +131,60 @@ def parse_knl_calls_and_average(knl: str, report: str) -> Tuple[int, float]:
     return calls, (total / calls if calls else 0.0)
 
 
+# kernels a library may launch ahead of the fused one within a call; their time belongs to it
+AUX_KERNELS = ("BindKnl", "OutlierKnl", "ScratchClearKnl")
+
+
+def _trace_files(report: str) -> List[str]:
+    if os.path.isfile(report):
+        return [report]
+    pats = [os.path.join(report, "**", "*kernel_trace.csv"), report + "*kernel_trace.csv"]
+    out: List[str] = []
+    for pat in pats:
+        out.extend(glob.glob(pat, recursive=True))
+    return sorted(set(out))
+
+
+def parse_knl_call_durations(knl: str, report: str, aux: Tuple[str, ...] = AUX_KERNELS) -> List[int]:
+    """Duration (ns) of every call, in the order of execution, from a rocprofv3
+    ``--kernel-trace`` output (``*_kernel_trace.csv`` at ``report``: a csv file, or a directory /
+    prefix that holds one).  A call is one dispatch of the kernel whose name is ``knl`` plus the
+    dispatches of the ``aux`` kernels that ran since the call before (the binding and outlier
+    kernels a library launches ahead of its fused kernel)."""
+    files = _trace_files(report)
+    if not files:
+        raise FileNotFoundError(f"no *kernel_trace.csv under {report}")
+    rows = []
+    for fname in files:
+        with open(fname, newline='') as f:
+            for row in csv.DictReader(f):
+                name = row.get("Kernel_Name", "")
+                if name == knl or name in aux:
+                    rows.append((int(row["Start_Timestamp"]), int(row["End_Timestamp"]), name))
+    rows.sort()
+    calls, pending = [], 0
+    for start, end, name in rows:
+        if name == knl:
+            calls.append(pending + end - start)
+            pending = 0
+        else:
+            pending += end - start
+    return calls
+
+
+def parse_knl_batch_times(knl: str, report: str, passes: int, skip_passes: int = 1) -> List[float]:
+    """For a program that ran the same sequence of batches ``passes`` times: per batch, the
+    median over the passes after the first ``skip_passes`` (warm-up: cold caches, clocks still
+    rising) of the call's duration in ns."""
+    calls = parse_knl_call_durations(knl, report)
+    if passes <= skip_passes or not calls or len(calls) % passes != 0:
+        raise ValueError(f"{len(calls)} calls of {knl} do not make {passes} passes "
+                         f"(of which {skip_passes} warm-up) over one sequence of batches")
+    n = len(calls) // passes
+    kept = np.asarray(calls, dtype=np.float64).reshape(passes, n)[skip_passes:]
+    return np.median(kept, axis=0).tolist()
+
+
 def parse_first_knl_total_time(report: str, reptype: str = "kernel_stats") -> int:
     """Total time (ns) of the kernel with the largest total time."""
     best = 0

@@ -8,6 +8,8 @@ its library is missing.  Names:
 ``cN_tuned``       CN with the schedules, occupancy and launch parameters recorded in
                    ``recflex_amd/tuned/cN_schedule.json`` (written by ``examples/tune.py``); the
                    default build if that file is absent
+``c1_o2``, ``c1_o5`` C1 built for 2 and 5 workgroups per CU (its light kernel reaches 8 by
+                   itself, so the dynamic-LDS pad has to hold the others off)
 ``c3_flat``        C3 with the flat tile walk instead of the XCD-segmented one (for comparison)
 ``c2s`` .. ``c5s``   shrunken C2..C5 (fewer rows / features / samples) that a CPU checker can follow
 ``variants``       one feature per (element type, dim, schedule candidate) over a spread of the
@@ -236,6 +238,8 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c3_tuned": lambda: _tuned(make_workload("C3"), "c3_schedule.json"),
     "c4_tuned": lambda: _tuned(make_workload("C4"), "c4_schedule.json"),
     "c5_tuned": lambda: _tuned(make_workload("C5"), "c5_schedule.json"),
+    "c1_o2": lambda: _default(make_workload("C1"), occupancy=2),
+    "c1_o5": lambda: _default(make_workload("C1"), occupancy=5),
     "c3_flat": lambda: _default(make_workload("C3"), xcd_aware=False),
     "c2s": lambda: _default(make_workload("C2", batch=512, max_rows=200_000)),
     "c3s": lambda: _default(make_workload("C3", batch=192, max_rows=60_000)),
@@ -303,7 +307,7 @@ def tune_fixture_dir() -> str:
     return os.path.join(MODELS_DIR, "tune_fixture")
 
 
-def make_fixture_tuner(model_dir: str, sample_batch_nums: int = 4):
+def make_fixture_tuner(model_dir: str, sample_batch_nums: int = 4, codegen_dir: str = None):
     from .schedules import SCHEDULE_MAPPING
     from .tuning import BasicConfig, Tuner
     from .utils import get_data_fnames
@@ -312,7 +316,7 @@ def make_fixture_tuner(model_dir: str, sample_batch_nums: int = 4):
                       data_fnames=get_data_fnames(data_dir),
                       schedule_config_fname=os.path.join(model_dir, "schedule_config.txt"),
                       table_config_fname=os.path.join(model_dir, "table_config.txt"),
-                      codegen_dir=tune_fixture_dir(), block_threads=BLOCK_THREADS,
+                      codegen_dir=codegen_dir or tune_fixture_dir(), block_threads=BLOCK_THREADS,
                       sample_batch_nums=sample_batch_nums)
     return Tuner(cfg, SCHEDULE_MAPPING)
 
@@ -358,3 +362,105 @@ def build_tune_fixture(model_dir: str) -> str:
     for choice in ("mean", "max"):
         tuner.compile_fixed_thread_binding(mix, choice, ablation._replace(remeasure=True))
     return tune_fixture_dir()
+
+
+# ------------------------------------------------------------------------------------------------
+# the global stage under rocprofv3: a 100-feature model whose fused kernel runs tens of
+# microseconds (C3 at half its batch, tables capped at 200 000 rows), default schedules, built
+# for two occupancies
+# ------------------------------------------------------------------------------------------------
+
+ROCPROF_FIXTURE_OCCUPANCIES = [2, 5]
+
+
+def rocprof_fixture_dir() -> str:
+    return os.path.join(MODELS_DIR, "tune_rocprof")
+
+
+def make_rocprof_tuner():
+    """Tuner over one seeded batch of the shrunken C3 (the arrays are regenerated from the seed
+    wherever this runs, and written to ``tune_rocprof/data`` for the profiled program)."""
+    from .schedules import SCHEDULE_MAPPING
+    from .tuning import BasicConfig, Tuner
+    from .workloads import gen_inputs
+    wl = make_workload("C3", batch=1024, max_rows=200_000)
+    indices, offsets = gen_inputs(wl._replace(seed=wl.seed + 7919))
+    cfg = BasicConfig(batch_sizes_fname="", data_fnames=[], schedule_config_fname="",
+                      table_config_fname="", codegen_dir=rocprof_fixture_dir(),
+                      block_threads=BLOCK_THREADS, sample_batch_nums=1)
+    templates = [ThreadPerBagSchedule, SubWavefrontPerBagSchedule, WavefrontPerBagSchedule,
+                 BlockPerBagSchedule]
+    return Tuner(cfg, SCHEDULE_MAPPING, batches=[[(i, o)] for i, o in zip(indices, offsets)],
+                 table_shapes=[(f.rows, f.dim) for f in wl.features],
+                 data_types=[f.data_type for f in wl.features],
+                 schedule_types=[templates for _ in wl.features])
+
+
+def rocprof_tune_config(**overrides):
+    return fixture_tune_config(occupancies=ROCPROF_FIXTURE_OCCUPANCIES, include_default=False,
+                               tile_bytes=0, **overrides)
+
+
+def build_rocprof_fixture() -> str:
+    """``tune_rocprof/all/o{2,5}``: the default mix as whole-model kernels, what
+    ``Tuner.tune_occupancy`` measures."""
+    import multiprocessing as mp
+    if mp.get_start_method(allow_none=True) != "spawn":
+        mp.set_start_method("spawn", force=True)
+    tuner = make_rocprof_tuner()
+    cfg = rocprof_tune_config(recompile=True)
+    mix = fixture_default_mix(tuner)
+    jobs = []
+    for occupancy in cfg.occupancies:
+        output_dir, build_dir = tuner.get_output_build_dir(-1, occupancy)
+        if tuner._build_full(output_dir, mix, occupancy, cfg):
+            jobs.append((output_dir, build_dir))
+    tuner._schedule_builds(jobs, cfg)
+    return rocprof_fixture_dir()
+
+
+# ------------------------------------------------------------------------------------------------
+# the compressed-model flow (examples/run_model.sh): one representative per cluster of like
+# features is tuned, the results are spread back over the full model
+# ------------------------------------------------------------------------------------------------
+
+def compress_fixture_dir() -> str:
+    return os.path.join(MODELS_DIR, "tune_compress")
+
+
+def build_compress_fixture(model_dir: str) -> str:
+    """``tune_compress/src``: the fixture model; ``tune_compress/model``: the same compressed by
+    ``examples/compress.py`` (its four like one-hot features become one), with the
+    reference-style local-stage kernels of its representatives built under
+    ``tune_compress/model/output``."""
+    import multiprocessing as mp
+    import shutil
+    import subprocess
+    import sys
+    if mp.get_start_method(allow_none=True) != "spawn":
+        mp.set_start_method("spawn", force=True)
+    root = compress_fixture_dir()
+    shutil.rmtree(root, ignore_errors=True)
+    # the fixture model with its like features described by one data_config line (features are
+    # clustered within a line): ``one-hot,1,c`` four times becomes ``one-hot,4,c``
+    src = os.path.join(root, "src")
+    shutil.copytree(model_dir, src)
+    merged: List[List[str]] = []
+    with open(os.path.join(model_dir, "data_config.txt")) as f:
+        for line in f:
+            fields = line.strip().split(",")
+            if len(fields) < 3:
+                continue
+            if merged and merged[-1][0] == fields[0] and merged[-1][2:] == fields[2:]:
+                merged[-1][1] = str(int(merged[-1][1]) + int(fields[1]))
+            else:
+                merged.append(fields)
+    with open(os.path.join(src, "data_config.txt"), "w") as f:
+        f.writelines(",".join(fields) + "\n" for fields in merged)
+    small = os.path.join(root, "model")
+    script = os.path.join(os.path.dirname(PACKAGE_DIR), "examples", "compress.py")
+    subprocess.run([sys.executable, script, "-m", src, "-o", small], check=True,
+                   stdout=subprocess.DEVNULL)
+    tuner = make_fixture_tuner(small, codegen_dir=os.path.join(small, "output"))
+    tuner.compile_local(fixture_tune_config(recompile=True, interference="replicate", occupancies=[4]))
+    return root

@@ -138,6 +138,9 @@ class FeatEmbed(nn.Module):
             torch.cuda.synchronize(self.device)
 
         self.output_units = self.lib.embed_dim_sum
+        # timing builds: (ticks before the first tile, ticks in all) summed over the workgroups
+        # of the last timed launch
+        self.last_workgroup_ticks = None
         self._io_cache_key = None
         self._io_bound = None
 
@@ -183,7 +186,9 @@ class FeatEmbed(nn.Module):
         if timing:
             if not self.lib.info.timing:
                 raise RuntimeError("timing=True needs a library emitted with timing=True")
-            times = torch.zeros([self.lib.num_features], dtype=torch.int64, device=self.device)
+            # per-feature ticks, then the workgroups' ticks before their first tile, then all
+            # of their ticks (kept in self.last_workgroup_ticks)
+            times = torch.zeros([self.lib.num_features + 2], dtype=torch.int64, device=self.device)
         if schedule_choice is not None:
             if schedule_choice.dtype != torch.int32 or schedule_choice.numel() != len(self.embed_tables) \
                     or schedule_choice.device.type != "cuda":
@@ -202,7 +207,9 @@ class FeatEmbed(nn.Module):
             if not timing_schedules or timing_schedules > n:
                 timing_schedules = n
             # device ticks (s_memtime) summed over the tiles of each schedule
-            task_times = times[:timing_schedules].cpu().to(torch.float64)
+            host_times = times.cpu().to(torch.float64)
+            task_times = host_times[:timing_schedules]
+            self.last_workgroup_ticks = (float(host_times[n]), float(host_times[n + 1]))
             return output, task_times
         return output
 

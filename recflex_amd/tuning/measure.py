@@ -326,10 +326,18 @@ def _run_script_args(table_config_fname: str, build_dir: str, data_dir: str,
     return args
 
 
+# the profiled program runs the sampled batches this many times; the first pass is warm-up and
+# the global stage takes each batch's median over the others (parser.parse_knl_batch_times)
+PROFILE_PASSES = 4
+PROFILE_WARMUP_PASSES = 1
+
+
 def rocprof_profile(table_config_fname: str, build_dir: str, data_dir: str, sample_batch_nums: int,
                     report_prefix: str, spec_feat_id: int = None, tile_bytes: int = 0,
-                    xcd_segments: int = 0, gpu_id: int = None) -> None:
-    """Leaves ``{report_prefix}_kernel_stats.csv`` (rocprofv3 ``--kernel-trace --stats``)."""
+                    xcd_segments: int = 0, passes: int = PROFILE_PASSES, gpu_id: int = None) -> None:
+    """Runs ``run_script.py`` on the built model as a child process under rocprofv3
+    (``--kernel-trace --stats``; the program itself stands right after ``--``) and leaves
+    ``{report_prefix}_kernel_stats.csv`` and ``{report_prefix}_kernel_trace.csv``."""
     if gpu_id is None:
         raise Exception("No valid GPU provided!")
     rocprof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
@@ -338,7 +346,8 @@ def rocprof_profile(table_config_fname: str, build_dir: str, data_dir: str, samp
     cmd = [rocprof, "--kernel-trace", "--stats", "--output-format", "csv", "-d", out_dir, "-o", name,
            "--"] + _run_script_args(table_config_fname, build_dir, data_dir, sample_batch_nums,
                                     spec_feat_id) + ["--tile_bytes", str(tile_bytes),
-                                                    "--xcd_segments", str(xcd_segments)]
+                                                    "--xcd_segments", str(xcd_segments),
+                                                    "--repeats", str(passes)]
     env = dict(os.environ)
     env["HIP_VISIBLE_DEVICES"] = str(gpu_id)
     env.setdefault("TMPDIR", "/tmp")

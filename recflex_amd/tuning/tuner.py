@@ -35,11 +35,11 @@ from recflex_amd.code_emitter.codegen import BAG_FIXED_BYTES, DEFAULT_TILE_BYTES
 from recflex_amd.utils import compile_build, os_check
 from recflex_amd.task_manager import TaskManager
 from recflex_amd.parser import (parse_raw_data_batches, parse_table_shapes, parse_table_dtypes,
-                                parse_schedule_types, parse_knl_total_time)
+                                parse_schedule_types, parse_knl_total_time, parse_knl_batch_times)
 
 from .measure import (measure_single_feat, rocprof_profile, measure_task_blocks,
                       measure_naive_candidate, measure_kernel_events, measure_tournament,
-                      save_batches, KernelTimer)
+                      save_batches, KernelTimer, PROFILE_PASSES, PROFILE_WARMUP_PASSES)
 
 
 class BasicConfig(NamedTuple):
@@ -655,7 +655,11 @@ class Tuner:
                           xcd_segments: int = 0) -> float:
         report_prefix = self._report_prefix(output_dir, tile_bytes, xcd_segments)
         if tune_config.profiler == "rocprofv3":
-            return parse_knl_total_time("FusedKnl", f"{report_prefix}_kernel_stats.csv")
+            # per batch the median over the measured passes of the call's kernels (the fused
+            # kernel and what the library launches ahead of it), summed over the batches: the
+            # same quantity the events timer reports
+            return float(sum(parse_knl_batch_times("FusedKnl", f"{report_prefix}_kernel_trace.csv",
+                                                   PROFILE_PASSES, PROFILE_WARMUP_PASSES)))
         with open(f"{report_prefix}.events.txt") as f:
             return float(f.read().strip())
 

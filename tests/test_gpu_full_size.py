@@ -107,6 +107,43 @@ def test_full_size_checksums(name):
     assert not bad, f"{len(bad)} features with wrong checksums, first {bad[:3]}"
 
 
+@pytest.mark.parametrize("name", ["c4_tuned", "c5_tuned"])
+def test_full_size_quantised_tables_match_oracle_on_a_sample(name):
+    """fp16 (C4) and int8 row-wise (C5) tables of N(0, 0.01) values at full size, where a rounding
+    problem at real bag lengths would show (the checksum tests use integer tables, which cannot
+    see one): every 16th feature over the whole batch and the first 64 bags of every feature
+    against the oracle (decode the row to fp32, then the fp32 sum), within 1e-3 relative or 1e-6
+    absolute.  Only the rows the sample looks up are copied back, so the largest tables need not
+    fit in host memory."""
+    import torch
+    from helpers import TOL, oracle
+    wl, dev, tables, indices, offsets, d_idx, d_off, layer = _setup(name)
+    assert wl.table_values == "normal" and wl.features[0].data_type in ("half", "int8")
+    out = layer.forward_indices(d_idx, d_off)
+    torch.cuda.synchronize()
+    col_of = np.concatenate([[0], np.cumsum([f.dim for f in wl.features])])
+    checked, worst, bad = 0, 0.0, []
+    for f, spec in enumerate(wl.features):
+        bags = wl.batch if f % 16 == 0 else 64
+        off = np.ascontiguousarray(offsets[f][:bags + 1])
+        idx = indices[f][:int(off[-1])]
+        # the looked-up rows only, bit for bit, under new row numbers
+        uniq, inv = np.unique(idx, return_inverse=True)
+        rows = tables[f].index_select(0, torch.from_numpy(uniq.astype(np.int64)).to(dev)).cpu().numpy()
+        want = oracle.pooled_sum_c([rows], [spec.dim], [spec.data_type], [inv.astype(np.int32)], [off])
+        got = out[:bags, col_of[f]:col_of[f + 1]].cpu().numpy()
+        rtol, atol = TOL[spec.data_type]
+        ok, max_abs, max_rel = oracle.within_tolerance(got, want, rtol, atol)
+        worst = max(worst, max_rel)
+        checked += bags * spec.dim
+        if not ok:
+            bad.append((f, spec, max_abs, max_rel))
+        if f % 50 == 0:
+            print(f"  feature {f} checked", flush=True)
+    print(f"  {checked} output elements checked, worst relative error beyond atol {worst:.2e}", flush=True)
+    assert not bad, f"{len(bad)} features out of tolerance, first {bad[:3]}"
+
+
 def test_launch_parameters_do_not_change_a_bit():
     """Tile size, grid size and the tile walk decide which workgroup sums a bag, never the order
     of the sum inside it: the full-size C3 output must be identical bit for bit."""

@@ -327,3 +327,34 @@ def test_outlier_tiles_are_switched_on_by_the_sampled_data():
     assert tuner.has_outlier_bags(fs)
     del tuner.batches
     assert not tuner.has_outlier_bags(fs)
+
+
+def test_kernel_trace_parser_groups_calls_and_takes_medians(tmp_path):
+    """rocprofv3 ``*_kernel_trace.csv``: a call is a FusedKnl dispatch plus the library's own
+    kernels launched ahead of it; per batch the median over the passes after the warm-up pass."""
+    from recflex_amd.parser import parse_knl_batch_times, parse_knl_call_durations
+    header = ('"Kind","Agent_Id","Queue_Id","Stream_Id","Thread_Id","Dispatch_Id","Kernel_Id","Kernel_Name",'
+              '"Correlation_Id","Start_Timestamp","End_Timestamp","LDS_Block_Size","Scratch_Size","VGPR_Count",'
+              '"Accum_VGPR_Count","SGPR_Count","Workgroup_Size_X","Workgroup_Size_Y","Workgroup_Size_Z",'
+              '"Grid_Size_X","Grid_Size_Y","Grid_Size_Z"')
+    rows, t = [], 1000
+    # 3 passes over 2 batches; pass 0 is slow (warm-up); an unrelated kernel in between
+    fused = [[900, 500], [100, 300], [120, 340]]
+    aux = [[50, 0], [10, 0], [30, 0]]             # OutlierKnl ahead of batch 0 only
+    for p in range(3):
+        for b in range(2):
+            if aux[p][b]:
+                rows.append(("OutlierKnl", t, t + aux[p][b])); t += aux[p][b] + 7
+            rows.append(("__amd_rocclr_copyBuffer", t, t + 40)); t += 47
+            rows.append(("FusedKnl", t, t + fused[p][b])); t += fused[p][b] + 7
+    body = "\n".join(f'"KERNEL_DISPATCH","Agent 1",1,0,8,{i},2,"{n}",{i},{s},{e},512,0,52,0,80,256,1,1,262144,1,1'
+                     for i, (n, s, e) in enumerate(reversed(rows)))      # file order is not time order
+    path = tmp_path / "report_kernel_trace.csv"
+    path.write_text(header + "\n" + body + "\n")
+    assert parse_knl_call_durations("FusedKnl", str(path)) == [950, 500, 110, 300, 150, 340]
+    assert parse_knl_call_durations("FusedKnl", str(tmp_path / "report")) == [950, 500, 110, 300, 150, 340]
+    assert parse_knl_batch_times("FusedKnl", str(path), passes=3, skip_passes=1) == [130.0, 320.0]
+    with pytest.raises(ValueError):
+        parse_knl_batch_times("FusedKnl", str(path), passes=4)
+    with pytest.raises(FileNotFoundError):
+        parse_knl_call_durations("FusedKnl", str(tmp_path / "nothing"))
