@@ -58,11 +58,19 @@ typedef struct recom_info {
   int32_t outliers;       /* 1 if emitted with outlier tiles: recom_process first launches a kernel
                            * that lists the bags too long for their feature's schedule, and the
                            * fused kernel runs them as tiles of their own, several workgroups each */
-  int32_t reserved[4];
+  int32_t static_workspace; /* 1 if the workspace fits the library's static device array, i.e.
+                             * recom_process_static_workspace can be used */
+  int32_t reserved[3];
 } recom_info;
 
-#define RECOM_ABI_VERSION 4     /* 4: the once-per-launch binding table of very wide models moved
-                                 * into the workspace */
+#define RECOM_ABI_VERSION 4     /* 4: recom_process_static_workspace; the once-per-launch binding
+                                 * table of very wide models moved into the workspace */
+
+/* largest workspace recom_process_static_workspace serves from the library's static array */
+#define RECOM_STATIC_WORKSPACE_MAX_BYTES (32 * 1024 * 1024)
+/* returned by recom_process_static_workspace of a library whose workspace is larger than that
+ * (negative: not a hipError_t) */
+#define RECOM_ESTATIC_WORKSPACE (-5)
 
 /* Static description of the emitted kernel.  No reference counterpart as a function: the
  * reference bakes the same numbers into process.cu (EMBED_DIM_SUM, block_threads,
@@ -184,6 +192,21 @@ typedef struct recom_process_args {
  * A library of more than 2048 features launches a one-workgroup kernel ahead
  * of the fused one that binds the model for this batch into a table in the workspace. */
 int recom_process(const recom_process_args *args);
+
+/* recom_process for callers that cannot allocate device memory at all, not even once: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Same arguments, same kernels, same result bits as
+ * recom_process, except that d_workspace / workspace_bytes are ignored: the workspace is a
+ * file-scope device array of the library (recom_get_workspace_bytes() bytes, at most
+ * RECOM_STATIC_WORKSPACE_MAX_BYTES; every device the library runs on holds its copy until the
+ * process ends).  A library that needs more returns RECOM_ESTATIC_WORKSPACE
+ * (recom_info.static_workspace == 0) and launches nothing.  Calls no hipMalloc / hipFree or
+ * other allocating routine; a small fill kernel ahead of the others puts the array's arrival
+ * counters and list header back to zero (no hipMemsetAsync, so the call can be captured).
+ * All calls of one library on one device share the one array: calls that may overlap (two
+ * streams, two threads) race and must be serialised by the caller.  A library whose
+ * recom_get_workspace_bytes() is 0 behaves exactly like recom_process. */
+int recom_process_static_workspace(const recom_process_args *args);
 
 /* ------------------------------------------------------------------------------------------
  * librecflex_host.so (CPU)

@@ -238,6 +238,11 @@ constexpr long long OUTLIER_BYTES = OUTLIERS ? (long long)sizeof(OutlierSpace) :
 constexpr long long BOUND_OFFSET = (SPLIT_BYTES + OUTLIER_BYTES + 255) / 256 * 256;
 constexpr long long BOUND_BYTES = BIND_ONCE ? (long long)sizeof(rfx::BoundTables<NUM_FEATS>) : 0LL;
 constexpr long long WORKSPACE_BYTES = BIND_ONCE ? BOUND_OFFSET + BOUND_BYTES : SPLIT_BYTES + OUTLIER_BYTES;
+// recom_process_static_workspace: the same workspace as a file-scope device array of the library
+constexpr long long STATIC_WORKSPACE_MAX = RECOM_STATIC_WORKSPACE_MAX_BYTES;
+constexpr bool STATIC_WORKSPACE_FITS = WORKSPACE_BYTES <= STATIC_WORKSPACE_MAX;
+constexpr long long STATIC_WORKSPACE_BYTES =
+    STATIC_WORKSPACE_FITS && WORKSPACE_BYTES > 0 ? WORKSPACE_BYTES : 256;
 static_assert(rfx::kBindMaxSplitTiles == {SPLIT_MAX_TILES} && rfx::kSplitGran == {SPLIT_GRANULARITY},
               "workspace regions were sized for this");
 
@@ -549,7 +554,7 @@ static int launch_kernels(const recom_process_args *a, void *workspace) {
   return static_cast<int>(e);
 }
 
-// checked before any HIP call
+// what both entry points check before any HIP call
 static bool valid_process_args(const recom_process_args *a) {
   if (!a || !a->d_embed_table_ptrs || !a->d_output || a->batch < 0 ||
       (!a->d_io_ptrs && (!a->d_arg_buffers || !a->d_arg_buffer_offsets)))
@@ -571,6 +576,76 @@ extern "C" int recom_process(const recom_process_args *a) {
     return static_cast<int>(hipErrorInvalidValue);
   if (a->batch == 0) return static_cast<int>(hipSuccess);
   return launch_kernels(a, WORKSPACE_BYTES > 0 ? a->d_workspace : nullptr);
+}
+
+// ---- the entry point that needs no caller workspace ----------------------------------------
+// The workspace as a file-scope device array: every device the library runs on holds its own
+// copy, at its own address, until the process ends.  In host code the name below is only a
+// handle for hipGetSymbolAddress; kernels and fills get the address that call returns.
+static __device__ __align__(256) char scratch[STATIC_WORKSPACE_BYTES];
+
+// Puts back to zero what a launch expects to find at zero in the workspace: the arrival
+// counters of every split-bag feature, and the header and the arrival counters of the outlier
+// list.  A fill kernel, not hipMemsetAsync, so that a caller may capture the call in a graph.
+extern "C" __global__ void __launch_bounds__(256) ScratchClearKnl(char *__restrict__ ws) {
+  const int first = blockIdx.x * blockDim.x + threadIdx.x, step = gridDim.x * blockDim.x;
+#if RFX_HAS_SPLIT
+  for (int f = blockIdx.y; f < NUM_FEATS; f += gridDim.y) {
+    if (c_split_region[f] < 0) continue;
+    const int dim = c_embed_dim_offsets[f + 1] - c_embed_dim_offsets[f];
+    int *counters = reinterpret_cast<int *>(ws) + c_split_region[f] +
+                    static_cast<long long>(rfx::kSplitMaxTiles) * dim;
+    for (int i = first; i < rfx::kSplitMaxTiles; i += step) counters[i] = 0;
+  }
+#endif
+#if RFX_OUTLIERS
+  if (blockIdx.y == 0) {
+    OutlierSpace *sp = reinterpret_cast<OutlierSpace *>(ws + SPLIT_BYTES);
+    int *hdr = reinterpret_cast<int *>(&sp->hdr);
+    for (int i = first; i < static_cast<int>(sizeof(rfx::OutlierHeader) / 4); i += step) hdr[i] = 0;
+    for (int i = first; i < OutlierSpace::kCap; i += step) sp->counters[i] = 0;
+  }
+#endif
+  (void)ws; (void)first; (void)step;
+}
+
+// device address of `scratch` on the current device, resolved once per device
+static hipError_t static_workspace_address(char **out) {
+  static char *addr[rfx::kMaxDevices];
+  static std::mutex mu;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= rfx::kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!addr[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    addr[dev] = static_cast<char *>(p);
+  }
+  *out = addr[dev];
+  return hipSuccess;
+}
+
+extern "C" int recom_process_static_workspace(const recom_process_args *a) {
+  if (!valid_process_args(a)) return static_cast<int>(hipErrorInvalidValue);
+  if (!STATIC_WORKSPACE_FITS) return RECOM_ESTATIC_WORKSPACE;
+  if (a->batch == 0) return static_cast<int>(hipSuccess);
+  if (WORKSPACE_BYTES == 0) return launch_kernels(a, nullptr);
+  char *ws = nullptr;
+  hipError_t e = static_workspace_address(&ws);
+  if (e != hipSuccess) return static_cast<int>(e);
+#if RFX_HAS_SPLIT || RFX_OUTLIERS
+  // the array keeps what the last call left in it
+  void *clear_args[] = {&ws};
+  const unsigned gy = static_cast<unsigned>(NUM_FEATS > 64 ? 64 : NUM_FEATS);
+  e = hipLaunchKernel(reinterpret_cast<const void *>(ScratchClearKnl), dim3(8, gy), dim3(256),
+                      clear_args, 0, static_cast<hipStream_t>(a->stream));
+  if (e != hipSuccess) return static_cast<int>(e);
+#endif
+  return launch_kernels(a, ws);
 }
 '''
 
@@ -627,6 +702,7 @@ extern "C" int recom_get_info(recom_info *out) {
   out->num_candidates = NUM_CANDIDATES;
   out->xcd_segments = XCD_SEGMENTS;
   out->outliers = OUTLIERS ? 1 : 0;
+  out->static_workspace = STATIC_WORKSPACE_FITS ? 1 : 0;
   return 0;
 }
 

@@ -27,7 +27,8 @@ class RecomInfo(ctypes.Structure):
         ("num_candidates", ctypes.c_int32),
         ("xcd_segments", ctypes.c_int32),
         ("outliers", ctypes.c_int32),
-        ("reserved", ctypes.c_int32 * 4),
+        ("static_workspace", ctypes.c_int32),
+        ("reserved", ctypes.c_int32 * 3),
     ]
 
 
@@ -62,9 +63,12 @@ class RecomProcessArgs(ctypes.Structure):
 
 
 RECOM_ABI_VERSION = 4
+RECOM_STATIC_WORKSPACE_MAX_BYTES = 32 * 1024 * 1024
+RECOM_ESTATIC_WORKSPACE = -5
 EXPORTED_SYMBOLS = ("recom_get_info", "recom_get_feature_tables", "recom_get_candidate_counts",
                     "recom_get_launch_info", "recom_get_workspace_bytes",
-                    "recom_get_max_concurrent_blocks", "recom_process")
+                    "recom_get_max_concurrent_blocks", "recom_process",
+                    "recom_process_static_workspace")
 
 
 class RecomError(RuntimeError):
@@ -91,6 +95,8 @@ class RecomLib:
         self.lib.recom_get_max_concurrent_blocks.argtypes = [_I32P]
         self.lib.recom_process.restype = ctypes.c_int
         self.lib.recom_process.argtypes = [ctypes.POINTER(RecomProcessArgs)]
+        self.lib.recom_process_static_workspace.restype = ctypes.c_int
+        self.lib.recom_process_static_workspace.argtypes = [ctypes.POINTER(RecomProcessArgs)]
 
         self.info = RecomInfo()
         rc = self.lib.recom_get_info(ctypes.byref(self.info))
@@ -166,9 +172,25 @@ class RecomLib:
                 arg_buffers: int = 0, arg_buffer_offsets: int = 0, tile_bytes: int = 0,
                 grid_blocks: int = 0, xcd_segments: int = 0, schedule_choice: int = 0,
                 times: int = 0, stream: int = 0, output_row_stride: int = 0,
-                workspace: int = 0, workspace_bytes: int = 0) -> None:
+                workspace: int = 0, workspace_bytes: int = 0,
+                static_workspace: bool = False) -> None:
         """All pointer arguments are raw device addresses (``tensor.data_ptr()``).  Without a
-        ``workspace``, a library that needs one uses ``default_workspace()``."""
+        ``workspace``, a library that needs one uses ``default_workspace()``.
+        ``static_workspace=True`` calls ``recom_process_static_workspace`` instead: no workspace
+        is passed or allocated, the library uses its own static device array."""
+        if static_workspace:
+            args = RecomProcessArgs(table_ptrs or None, io_ptrs or None, arg_buffers or None,
+                                    arg_buffer_offsets or None, output or None, batch, tile_bytes,
+                                    grid_blocks, xcd_segments, schedule_choice or None,
+                                    times or None, stream or None, output_row_stride, None, 0)
+            rc = self.lib.recom_process_static_workspace(ctypes.byref(args))
+            if rc == RECOM_ESTATIC_WORKSPACE:
+                raise RecomError(f"recom_process_static_workspace: the library needs "
+                                 f"{self.workspace_bytes} bytes of workspace, its static array holds "
+                                 f"at most {RECOM_STATIC_WORKSPACE_MAX_BYTES};", rc)
+            if rc != 0:
+                raise RecomError("recom_process_static_workspace", rc)
+            return
         if not workspace and self.workspace_bytes:
             workspace, workspace_bytes = self.default_workspace(), self.workspace_bytes
         args = RecomProcessArgs(table_ptrs or None, io_ptrs or None, arg_buffers or None,
