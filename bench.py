@@ -4,12 +4,26 @@
 
 A step is one launch of the fused kernel over one batch of the synthetic workload whose inputs
 (tables, indices, offsets) and output buffer are already resident in HBM.  Prints ONE JSON line:
-``value`` is the achieved algorithmic bandwidth in GB/s of the headline workload (C3, the
-heterogeneous 100-feature configuration), next to kernel microseconds, pooled lookups per second,
-the roofline object for ``FusedKnl`` and the CPU baseline (the oracle: per-feature torch
-``embedding_bag(mode="sum")`` + concat on the host cores) timed in the same run, which is also
-the correctness check of the GPU result.  ``--also`` adds the same figures for further
-configurations under ``"configs"``.
+``value`` is the whole-job rate of the headline workload (C3, the heterogeneous 100-feature
+configuration) in algorithmic GB/s -- the bytes the path delivers (rows + indices + offsets +
+output, a row counted as often as it is looked up) over the wall time of the K timed steps --
+next to kernel microseconds, pooled lookups per second, the roofline object for ``FusedKnl``
+and the CPU baseline (the oracle: per-feature torch ``embedding_bag(mode="sum")`` + concat on
+the host cores) timed in the same run, which is also the correctness check of the GPU result.
+``--also`` adds the same figures for further configurations under ``"configs"``.
+
+Three byte counts per launch, because Zipf-hot rows are served from the caches:
+
+* ``algorithmic_bytes``: every lookup's row counted (what a cache-less device would move); the
+  rate it gives (``algorithmic_gbps``) can exceed the HBM peak and is not a roofline fraction;
+* ``compulsory_bytes``: every distinct 128-byte line of the touched rows once, plus indices,
+  offsets and output -- what must cross the HBM pins even with perfect caches, computed live;
+* ``hbm_traffic_bytes``: what did cross them (rocprofv3 FETCH_SIZE / WRITE_SIZE, recorded in
+  ``recflex_amd/tuned/hbm_traffic.json`` for the library it was measured on; ``null`` when the
+  library in use is not that one).
+
+``roofline.frac`` = HBM bytes per launch / kernel time / 8 TB/s, with the measured traffic where
+it is known and the compulsory bytes (a lower bound of the traffic) otherwise; it cannot exceed 1.
 """
 
 import argparse
@@ -25,10 +39,6 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0   # MI355X, HBM3E, published
 METRIC = "fused-kernel \u00b5s + achieved HBM GB/s (% of MI355X peak) per model config"
 
-# HBM bytes per launch (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, rocprofv3 --pmc, scale factors
-# from a 1 GiB copy in the same runs) of the tuned models, as recorded in
-# profiles/FusedKnl_c2_c3_c4_c5.md; a live run cannot read these counters itself.
-MEASURED_TRAFFIC_BYTES = {"c3_tuned": 552.4e6, "c2_tuned": 44.5e6, "c4_tuned": 22477e6, "c5_tuned": 7290e6}
 
 TOL = {"float": (1e-5, 1e-6), "half": (1e-3, 1e-6), "int8": (1e-3, 1e-6)}
 
@@ -164,7 +174,8 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
     import torch
     from recflex_amd import prebuilt
     from recflex_amd.rec_modules import FeatEmbed
-    from recflex_amd.workloads import algorithmic_bytes, gen_inputs, gen_tables
+    from recflex_amd.hbm_traffic import recorded_traffic_bytes
+    from recflex_amd.workloads import algorithmic_bytes, compulsory_bytes, gen_inputs, gen_tables
 
     model = pick_model(name)
     spec = prebuilt.model_spec(model)
@@ -187,6 +198,9 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
 
     lookups = [len(i) for i in indices]
     alg_bytes = algorithmic_bytes(wl, lookups)
+    comp_bytes = compulsory_bytes(wl, indices, offsets)
+    # HBM bytes per launch as the counters gave them, if they were taken on this very library
+    traffic = recorded_traffic_bytes(model)
 
     bound = layer.bind_inputs(d_idx, d_off)      # inputs validated, address table uploaded: once
     run = lambda: layer.forward_indices(bound, tile_bytes=tile_bytes, grid_blocks=grid_blocks,
@@ -217,16 +231,26 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
     kernel_us_avg = sum(durs) / len(durs)
     kernel_us_med = durs[len(durs) // 2]
 
+    kernel_s = kernel_us_avg * 1e-6
+    hbm_bytes = traffic if traffic is not None else comp_bytes
     res = {
         "workload": name, "model": model, "features": wl.num_features, "batch": wl.batch,
         "embed_dim_sum": wl.embed_dim_sum, "lookups": int(sum(lookups)),
         "table_gb": round(wl.table_bytes() / 1e9, 2),
-        "algorithmic_bytes": int(alg_bytes),
+        "algorithmic_bytes": int(alg_bytes), "compulsory_bytes": int(comp_bytes),
+        "hbm_traffic_bytes": traffic,
+        "traffic_over_compulsory": (traffic / comp_bytes) if traffic is not None else None,
         "ms_per_step": wall / steps * 1e3,
         "kernel_us_avg": kernel_us_avg, "kernel_us_median": kernel_us_med,
-        "lookups_per_s": sum(lookups) / (kernel_us_avg * 1e-6),
-        "achieved_gbps": alg_bytes / (kernel_us_avg * 1e-6) / 1e9,
-        "pct_of_peak": alg_bytes / (kernel_us_avg * 1e-6) / 1e9 / HBM_PEAK_GBPS * 100.0,
+        "lookups_per_s": sum(lookups) / kernel_s,
+        # whole-job rate: the K timed steps by the wall clock
+        "job_algorithmic_gbps": alg_bytes / (wall / steps) / 1e9,
+        # by the kernel's own duration
+        "algorithmic_gbps": alg_bytes / kernel_s / 1e9,
+        "compulsory_gbps": comp_bytes / kernel_s / 1e9,
+        "hbm_gbps": hbm_bytes / kernel_s / 1e9,
+        "hbm_basis": "hbm_counters" if traffic is not None else "compulsory_bytes",
+        "frac_of_hbm_peak": hbm_bytes / kernel_s / 1e9 / HBM_PEAK_GBPS,
         "bodies": layer.lib.info.num_bodies, "occupancy": layer.lib.info.occupancy,
         "grid_blocks": grid_blocks or layer.max_concurrent_blocks,
         "setup_s": round(setup_s, 2),
@@ -293,7 +317,7 @@ def main():
 
     line = {
         "metric": METRIC,
-        "value": head["achieved_gbps"],
+        "value": head["job_algorithmic_gbps"],
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -309,14 +333,21 @@ def main():
                                f"{head['lookups']} lookups, {head['table_gb']} GB of tables",
                    "build": head["model"], "bodies": head["bodies"],
                    "occupancy": head["occupancy"], "grid_blocks": head["grid_blocks"]},
+        "value_definition": "algorithmic bytes per launch (rows + int32 indices + int32 offsets + fp32 "
+                            "output, a row counted once per lookup) / wall time per step",
         "kernel_us": head["kernel_us_avg"],
         "kernel_us_median": head["kernel_us_median"],
         "lookups_per_s": head["lookups_per_s"],
-        "pct_of_peak": head["pct_of_peak"],
-        "roofline": {"bound": "hbm", "achieved": head["achieved_gbps"], "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": head["achieved_gbps"] / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(head["model"]), "kernel": "FusedKnl",
-                     "algorithmic_bytes_per_launch": head["algorithmic_bytes"]},
+        # achieved = bytes that crossed the HBM pins per launch / FusedKnl's duration: the
+        # counters' figure where it was taken on this library, else the compulsory bytes (every
+        # distinct memory line once), which the traffic cannot be below; never above the peak
+        "roofline": {"bound": "hbm", "achieved": head["hbm_gbps"], "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": head["frac_of_hbm_peak"], "basis": head["hbm_basis"],
+                     "traffic": head["hbm_traffic_bytes"], "kernel": "FusedKnl",
+                     "compulsory_bytes_per_launch": head["compulsory_bytes"],
+                     "traffic_over_compulsory": head["traffic_over_compulsory"],
+                     "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
+                     "algorithmic_gbps": head["algorithmic_gbps"]},
     }
     if "gather_floor_us" in head:
         # time of the bare fetch of the same rows (gather probe): what the memory system allows

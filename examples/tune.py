@@ -36,7 +36,7 @@ from schedules.warp_per_sample import WarpPerSampleSchedule, WarpPerSampleParams
 from schedules.one_hot import OneHotSchedule, OneHotParams
 from schedules.one_hot_multi_block import OneHotMultiBlockSchedule, OneHotMultiBlockParams
 from recflex_amd.schedules import (ThreadPerBagSchedule, SubWavefrontPerBagSchedule,
-                                   WavefrontPerBagSchedule, BlockPerBagSchedule)
+                                   WavefrontPerBagSchedule, BlockPerBagSchedule, OneHotBagSchedule)
 
 # number of compute units and resident threads per CU of an MI355X, used when a run only
 # compiles and no device can be queried
@@ -122,7 +122,11 @@ def create_tuner(args: argparse.Namespace) -> Tuner:
         return Tuner(basic_config, schedule_mapping=globals(), batches=batches,
                      table_shapes=[(f.rows, f.dim) for f in wl.features],
                      data_types=[f.data_type for f in wl.features],
-                     schedule_types=[all_templates() for _ in wl.features])
+                     # the row-copy template only where no sampled bag holds more than one lookup
+                     schedule_types=[all_templates() + ([OneHotBagSchedule] if
+                                                        max(int(np.diff(o).max()) for _, o in batches[f]) <= 1
+                                                        else [])
+                                     for f in range(wl.num_features)])
 
     model_dir = args.model_dir
     data_dir = os.path.join(model_dir, "data")

@@ -224,6 +224,7 @@ constexpr bool TIMING = {"true" if timing else "false"};
 constexpr bool STATIC_BINDING = {"true" if fixed_task_block_nums else "false"};
 #define RFX_BIND_ONCE {1 if bind_once else 0}
 constexpr bool BIND_ONCE = RFX_BIND_ONCE;
+static_assert(rfx::kBindKeepAddrs == 512, "the emitter decides by this where a tile finds its addresses");
 // bytes of workspace the split-bag schedules need (0: no schedule splits bags)
 constexpr long long SPLIT_BYTES = {workspace_floats * 4}LL;
 #define RFX_HAS_SPLIT {1 if workspace_floats > 0 else 0}
@@ -264,7 +265,8 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
     const int {vars_.bag_begin}, const int {vars_.bag_end},
     char *__restrict__ {vars_.shmem}, rfx::f32x4 *__restrict__ {vars_.stage},
     const int {vars_.split_part}, const int {vars_.split_parts},
-    float *__restrict__ {vars_.split_region}, const int {vars_.skip_long}) {{
+    float *__restrict__ {vars_.split_region}, const int {vars_.skip_long},
+    const int {vars_.one_per_bag}) {{
   {schedule.EmitScheduleBody(params)}
 }}
 '''
@@ -352,7 +354,8 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
         call_args = (f"table, indices, offsets, d_output, {vars_.out_row_stride}, embed_dim_offset, "
                      f"{vars_.bag_begin}, {vars_.bag_end}, reinterpret_cast<char *>(&s), "
                      + ("&s_stage.seg[0][0]" if need_stage else "nullptr")
-                     + f", {vars_.split_part}, {vars_.split_parts}, {vars_.split_region}, {vars_.skip_long}")
+                     + f", {vars_.split_part}, {vars_.split_parts}, {vars_.split_region}, {vars_.skip_long}"
+                     + f", {vars_.one_per_bag}")
         cases = "".join(
             f"      case {feat_idx}: ProcessFeat{feat_idx}({call_args}); break;\n"
             for feat_idx in body_ids)
@@ -366,9 +369,10 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
             bound_src = "d_bound->"
         else:
             bind_decl = "  __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;\n"
-            bind_call = (f"  const int regular_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}, HAS_SPLIT>(\n"
+            bind_call = (f"  const int regular_tiles = rfx::bind_tiles<NUM_FEATS, {vars_.BLOCK_THREADS}, HAS_SPLIT,\n"
+                         "                                            NUM_CANDIDATES == NUM_FEATS>(\n"
                          "      s_bind, io, tile_bytes, c_lookup_bytes, c_bag_bytes, c_cand_begin, c_cand_gran,\n"
-                         f"      d_schedule_choice, {fixed_arg}, gridDim.x);\n  (void)d_bound;")
+                         f"      d_schedule_choice, {fixed_arg}, gridDim.x, d_embed_table_ptrs);\n  (void)d_bound;")
             bound_src = "s_bind."
         bind_kernel = f'''
 // One workgroup binds the whole model for this launch (models of thousands of features).
@@ -424,6 +428,19 @@ extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
   __syncthreads();
   if (threadIdx.x == 0) rfx::outliers_done(d_outliers);
 ''' if outliers else ''
+        # rfx::kBindKeepAddrs: the binding of a model of up to 512 features keeps every feature's
+        # table / indices / offsets address in LDS, and whether the batch holds one lookup per bag
+        keep_addrs = not bind_once and num_feats <= 512
+        feature_addrs = f'''    // the feature's addresses, which the binding kept in LDS
+    const char *table = rfx::global_ptr<char>(rfx::uniform64(s_bind.table_addr[feat_idx]));
+    const int *indices = rfx::global_ptr<int>(rfx::uniform64(s_bind.indices_addr[feat_idx]));
+    const int *offsets = rfx::global_ptr<int>(rfx::uniform64(s_bind.offsets_addr[feat_idx]));
+    const int {vars_.one_per_bag} = __builtin_amdgcn_readfirstlane(s_bind.one_per_bag[feat_idx]);
+''' if keep_addrs else f'''    const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[feat_idx]);
+    const int *indices = io.indices(feat_idx);
+    const int *offsets = io.offsets(feat_idx);
+    const int {vars_.one_per_bag} = 0;
+'''
         kernel = bind_kernel + outlier_kernel + f'''
 extern "C" __global__ void {launch_bounds} FusedKnl(
     const int64_t *__restrict__ d_embed_table_ptrs,
@@ -466,7 +483,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
       if (tile >= total_tiles) continue;
     }}
 {outlier_tile}{timing_begin if timing and timing_branch else ''}
-    const int feat_idx = __builtin_amdgcn_readfirstlane(rfx::find_feature<NUM_FEATS>(s_bind.prefix, tile));
+    const int feat_idx = __builtin_amdgcn_readfirstlane(rfx::find_feature_wave<NUM_FEATS>(s_bind.prefix, tile));
     const int bags_per_tile = {bound_src}bags_per_tile[feat_idx];
     int {vars_.bag_begin} = (tile - s_bind.prefix[feat_idx]) * bags_per_tile;
     int {vars_.bag_end} = min(batch, {vars_.bag_begin} + bags_per_tile);
@@ -484,10 +501,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
       }}
       {vars_.split_region} = d_workspace + {"c_split_region[feat_idx]" if has_split else "0"};
     }}
-    const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[feat_idx]);
-    const int *indices = io.indices(feat_idx);
-    const int *offsets = io.offsets(feat_idx);
-    const int embed_dim_offset = c_embed_dim_offsets[feat_idx];
+{feature_addrs}    const int embed_dim_offset = c_embed_dim_offsets[feat_idx];
     const int {vars_.skip_long} = {"outlier_tiles > 0 && c_long_thr[feat_idx] > 0 ? c_long_thr[feat_idx] : 0x7fffffff" if outliers else "0x7fffffff"};
 {timing_begin if timing and not timing_branch else ''}
     switch (c_cand_func_ids[{bound_src}cand[feat_idx]]) {{

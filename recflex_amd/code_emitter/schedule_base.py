@@ -115,6 +115,10 @@ class ScheduleVars(NamedTuple):
     # int: bags of more lookups than this were found ahead of the kernel and run as tiles of
     # their own, the body must leave them alone (INT_MAX when there are none)
     skip_long: str = "skip_longer_than"
+    # int: 1 if this batch holds exactly as many lookups of the feature as bags (every bag may
+    # have exactly one lookup; a body for such bags can fetch indices[bag] ahead of the bag's
+    # offsets and check afterwards), else 0
+    one_per_bag: str = "one_per_bag"
     split_part: str = "split_part"
     split_parts: str = "split_parts"
     split_region: str = "split_region"

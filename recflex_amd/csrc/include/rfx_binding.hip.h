@@ -39,15 +39,30 @@ struct IoView {
   const int64_t *__restrict__ arg_offsets;
   int batch;
 
-  __device__ __forceinline__ const int *offsets(int f) const {
-    if (io_ptrs) return global_ptr<int>(io_ptrs[2 * f + 1]);
-    return global_ptr<int>(reinterpret_cast<int64_t>(arg_base) + arg_offsets[f]);
+  __device__ __forceinline__ int64_t offsets_addr(int f) const {
+    if (io_ptrs) return io_ptrs[2 * f + 1];
+    return reinterpret_cast<int64_t>(arg_base) + arg_offsets[f];
   }
-  __device__ __forceinline__ const int *indices(int f) const {
-    if (io_ptrs) return global_ptr<int>(io_ptrs[2 * f]);
-    return global_ptr<int>(reinterpret_cast<int64_t>(arg_base) + arg_offsets[f] +
-                           alignmem((static_cast<int64_t>(batch) + 1) * 4));
+  __device__ __forceinline__ int64_t indices_addr(int f) const {
+    if (io_ptrs) return io_ptrs[2 * f];
+    return reinterpret_cast<int64_t>(arg_base) + arg_offsets[f] +
+           alignmem((static_cast<int64_t>(batch) + 1) * 4);
   }
+  // Both addresses of feature f from two independent loads of one cache line, whichever form the
+  // inputs have (no branch: the binding issues these loads for all features at once).
+  __device__ __forceinline__ void addrs(int f, int64_t &indices_at, int64_t &offsets_at) const {
+    typedef long long pair_t __attribute__((ext_vector_type(2), aligned(8)));
+    const bool ptrs = io_ptrs != nullptr;
+    // pointer table: {indices, offsets} of f; packed form: {byte offset of f, of f + 1}
+    const int64_t *src = ptrs ? io_ptrs + 2 * f : arg_offsets + f;
+    const pair_t ab = *reinterpret_cast<const pair_t *>(src);
+    const int64_t a = ab.x, b = ab.y;
+    const int64_t base = reinterpret_cast<int64_t>(arg_base);
+    offsets_at = ptrs ? b : base + a;
+    indices_at = ptrs ? a : base + a + alignmem((static_cast<int64_t>(batch) + 1) * 4);
+  }
+  __device__ __forceinline__ const int *offsets(int f) const { return global_ptr<int>(offsets_addr(f)); }
+  __device__ __forceinline__ const int *indices(int f) const { return global_ptr<int>(indices_addr(f)); }
 };
 
 // Schedules that split a bag over several workgroups (rfx::split_bags) announce themselves with
@@ -77,29 +92,84 @@ constexpr int kBindMaxSplitTiles = 2048;
 // most this many times the target traffic per tile
 constexpr int kMaxTileFactor = 8;
 
+// Models of up to this many features also keep, per feature, the three addresses a tile needs
+// (table, indices, offsets) in LDS: the binding reads them anyway, and a tile then starts with
+// an LDS read instead of a round trip to memory for its pointers.
+constexpr int kBindKeepAddrs = 512;
+
 template <int F> struct BindingStorage {
+  static constexpr bool kKeepAddrs = F <= kBindKeepAddrs;
   int prefix[F + 1];      // prefix[f] = first global tile id of feature f
   int bags_per_tile[F];
   int cand[F];            // index (into the candidate tables) of the schedule feature f runs
   long long partial[16];  // per-wavefront sums of the batch's traffic (automatic tile size)
+  int64_t table_addr[kKeepAddrs ? F : 1];
+  int64_t indices_addr[kKeepAddrs ? F : 1];
+  int64_t offsets_addr[kKeepAddrs ? F : 1];
+  // 1: the batch holds exactly as many lookups of this feature as bags (every bag may have
+  // exactly one: bodies for bags of one lookup then fetch indices[bag] without waiting for the
+  // bag's offsets, and check afterwards)
+  unsigned char one_per_bag[kKeepAddrs ? F : 1];
 };
+
+// a 64-bit value that is the same in every lane, as a scalar
+__device__ __forceinline__ int64_t uniform64(const int64_t v) {
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<int>(v));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<int>(v >> 32));
+  return static_cast<int64_t>((static_cast<unsigned long long>(hi) << 32) | lo);
+}
 
 // Automatic tile size (tile_bytes <= 0): the batch's traffic divided by kAutoTilesPerWorkgroup
 // tiles for each workgroup of the grid, within [kAutoTileMin, kAutoTileMax], in steps of 4 KiB.
 // Small batches keep 64 KiB tiles; a batch of tens of GB with bags of hundreds of wide rows gets
 // 256 KiB, several bags per tile instead of one (measured on the 400-feature fp16 model with its
 // default schedules: 7.1 ms with 64 KiB tiles, 5.0 ms with 256 KiB).
+// A batch too small for that (less than kAutoTileMin of traffic per workgroup of the grid) gets
+// about two tiles per workgroup instead, down to kAutoTileFloor: its launch is a matter of
+// latencies -- every pass of a workgroup over a tile is a chain of dependent round trips to
+// memory -- so the passes are spread over all workgroups as evenly as their number allows
+// (measured on 26 features x 4 096 one-lookup bags, 1 024 workgroups: 9.0 us with 54 KiB tiles
+// of two passes each, 8.3 us with 32 KiB tiles of one).
 constexpr int kAutoTilesPerWorkgroup = 64;
 constexpr int kAutoTileMin = 64 * 1024;
 constexpr int kAutoTileMax = 256 * 1024;
+constexpr int kAutoTileFloor = 4 * 1024;
 
+__host__ __device__ inline int auto_tile_size(const long long total, const int grid_blocks) {
+  const long long grid = grid_blocks > 0 ? grid_blocks : 1;
+  long long t = total / (grid * kAutoTilesPerWorkgroup);
+  if (t >= kAutoTileMin) return static_cast<int>(t > kAutoTileMax ? kAutoTileMax : t) & ~4095;
+  t = total / (2 * grid);
+  t = t < kAutoTileFloor ? kAutoTileFloor : (t > kAutoTileMin ? kAutoTileMin : t);
+  return static_cast<int>(t) & ~1023;
+}
+
+// Inclusive prefix sum over the 64 lanes of a wavefront with DPP moves (no LDS traffic): shifts
+// by 1, 2, 4 and 8 inside each row of 16 lanes (lanes shifted in from outside the row read 0),
+// then lane 15 of a row broadcast to the next row (rows 1 and 3), then lane 31 to rows 2 and 3.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ int dpp_or_zero(const int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
 __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const int t = __shfl_up(v, d, 64);
-    if (lane >= d) v += t;
-  }
+  (void)lane;
+  v += dpp_or_zero<0x111, 0xf>(v);   // row_shr:1
+  v += dpp_or_zero<0x112, 0xf>(v);   // row_shr:2
+  v += dpp_or_zero<0x114, 0xf>(v);   // row_shr:4
+  v += dpp_or_zero<0x118, 0xf>(v);   // row_shr:8
+  v += dpp_or_zero<0x142, 0xa>(v);   // row_bcast:15 -> rows 1, 3
+  v += dpp_or_zero<0x143, 0xc>(v);   // row_bcast:31 -> rows 2, 3
   return v;
+}
+// Sum of v over the wavefront, the same value in every lane (the same steps on floats; the order
+// of the additions is fixed, so every wavefront of every workgroup gets the same bits).
+__device__ __forceinline__ float wave_sum(float v) {
+  v += __int_as_float(dpp_or_zero<0x111, 0xf>(__float_as_int(v)));
+  v += __int_as_float(dpp_or_zero<0x112, 0xf>(__float_as_int(v)));
+  v += __int_as_float(dpp_or_zero<0x114, 0xf>(__float_as_int(v)));
+  v += __int_as_float(dpp_or_zero<0x118, 0xf>(__float_as_int(v)));
+  v += __int_as_float(dpp_or_zero<0x142, 0xa>(__float_as_int(v)));
+  v += __int_as_float(dpp_or_zero<0x143, 0xc>(__float_as_int(v)));
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 // lookup_bytes[f]: bytes fetched per lookup (row + index); bag_bytes[f]: bytes per bag that do
@@ -113,115 +183,178 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
 // fixed_tiles: if non-null, the tile count per feature is taken from it instead of from the
 // live offsets (static thread binding, for the ablation).
 // grid_blocks: workgroups of the fused kernel's grid (for the automatic tile size).
+// table_ptrs: the tables' base addresses, kept in LDS beside the input addresses for models of
+// up to kBindKeepAddrs features (required for those, not read otherwise).
+// ONE_CAND: every feature has exactly one candidate (a production build): feature f runs
+// candidate f and the candidate tables are not read to find that out.
 // Returns the total number of tiles.  Ends with a barrier.
-template <int F, int BT, bool SPLIT = false>
+//
+// Tile counts come from quotients of traffic figures; those are taken in single precision (a
+// 64-bit integer division costs some hundred instructions, and every workgroup of every launch
+// pays for the binding before its first load).  Being off by one tile near a boundary changes
+// nothing but the balance, and every workgroup computes the same figures.  The divisions that
+// decide which bags a tile holds stay exact.
+__device__ __forceinline__ long long approx_ceil_div(const long long a, const long long b) {
+  const float q = static_cast<float>(a) / static_cast<float>(b);
+  return static_cast<long long>(ceilf(q));
+}
+
+template <int F, int BT, bool SPLIT = false, bool ONE_CAND = false>
 __device__ __forceinline__ int
 bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
            const int *__restrict__ lookup_bytes, const int *__restrict__ bag_bytes,
            const int *__restrict__ cand_begin, const int *__restrict__ cand_gran,
            const int *__restrict__ choice, const int *__restrict__ fixed_tiles,
-           const int grid_blocks) {
+           const int grid_blocks, const int64_t *__restrict__ table_ptrs = nullptr) {
   static_assert(BT <= 16 * 64, "partial sums: at most 16 wavefronts");
   const int tid = threadIdx.x;
   const int B = io.batch;
+  // this thread is responsible for features tid, tid + BT, ...
+  constexpr int K = (F + BT - 1) / BT;
+  // up to 64 features: all of them sit in the first wavefront, which then needs no LDS and no
+  // barrier to add up the traffic and to scan the tile counts
+  constexpr bool ONE_WAVE = F <= 64;
+  long long cost[K];        // traffic of the feature in this batch
+  int gran[K];              // bags per workgroup pass of the feature's schedule (kSplitGran: splits)
 
-  // tiles of every feature this thread is responsible for (tid, tid + BT, ...) at the given
-  // tile size; returns the traffic of those features
-  // split_unit: traffic per part of a split bag (0: no bag is split)
-  auto bind_features = [&](const int tile_size, const long long split_unit) {
-    long long traffic = 0;
-    for (int f = tid; f < F; f += BT) {
+  // Step 1, the only one that reads memory, in two rounds of loads: the addresses, the schedule
+  // and the per-lookup / per-bag bytes of every feature; then its live lookup count.
+  int64_t offs_at[K], idx_at[K], table_at[K];
+  int lookup_b[K], bag_b[K], cand[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    // surplus threads repeat the last feature, stores included: no branch stands between the
+    // loads of this step
+    const int f = min(tid + k * BT, F - 1);
+    io.addrs(f, idx_at[k], offs_at[k]);
+    table_at[k] = 0;
+    if constexpr (BindingStorage<F>::kKeepAddrs) table_at[k] = table_ptrs[f];
+    cand[k] = f;
+    if constexpr (!ONE_CAND) {
       const int first = cand_begin[f];
       const int ncand = cand_begin[f + 1] - first;
       int pick = choice ? choice[f] : 0;
       pick = pick < 0 ? 0 : (pick >= ncand ? ncand - 1 : pick);
-      s.cand[f] = first + pick;
-      int g = cand_gran[first + pick];
-      const bool may_split = g == kSplitGran && !fixed_tiles;
-      if (g == kSplitGran) g = 1;
-      int64_t want;
-      int64_t bag_cost = 0;       // mean traffic of one bag of this feature
-      if (fixed_tiles) {
-        want = fixed_tiles[f];
-      } else {
-        const int *offs = io.offsets(f);
-        const int64_t lookups = static_cast<int64_t>(offs[B]) - offs[0];
-        const int64_t cost = lookups * lookup_bytes[f] + static_cast<int64_t>(B) * bag_bytes[f];
-        traffic += cost;
-        want = (cost + tile_size - 1) / tile_size;
-        bag_cost = B > 0 ? cost / B : 0;
-      }
-      int tiles = want < 1 ? 1 : (want > B ? B : static_cast<int>(want));
-      int bpt = 0;
-      int64_t parts = 1;
-      if (SPLIT && may_split && B > 0 && split_unit > 0 && bag_cost > 2 * split_unit) {
-        parts = (bag_cost + split_unit - 1) / split_unit;
-        if (parts > kBindMaxParts) parts = kBindMaxParts;
-        if (parts * B > kBindMaxSplitTiles) parts = kBindMaxSplitTiles / B;
-      }
-      if (parts > 1) {
-        tiles = B * static_cast<int>(parts);
-        bpt = -static_cast<int>(parts);
-      } else if (B > 0) {
-        bpt = (B + tiles - 1) / tiles;
-        // Tiles are whole workgroup passes (g bags) -- unless one pass of this schedule is more
-        // than kMaxTileFactor times the traffic a tile should carry: then the tile keeps its
-        // share of the traffic and some of the schedule's teams idle.
-        const int whole = (bpt + g - 1) / g * g;
-        if (fixed_tiles || bpt >= g ||
-            static_cast<int64_t>(whole) * bag_cost <= static_cast<int64_t>(kMaxTileFactor) * tile_size)
-          bpt = whole;
-        tiles = (B + bpt - 1) / bpt;
-      } else {
-        tiles = 0;
-      }
-      s.bags_per_tile[f] = bpt;
-      s.prefix[f + 1] = tiles;
+      cand[k] = first + pick;
     }
-    return traffic;
-  };
+    gran[k] = cand_gran[cand[k]];
+    lookup_b[k] = lookup_bytes[f];
+    bag_b[k] = bag_bytes[f];
+  }
+  float traffic = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const bool real = tid + k * BT < F;
+    const int f = min(tid + k * BT, F - 1);
+    cost[k] = 0;
+    bool one_per_bag = false;
+    if (!fixed_tiles) {
+      const int *offs = global_ptr<int>(offs_at[k]);
+      const int first_lookup = offs[0];
+      const int64_t lookups = static_cast<int64_t>(offs[B]) - first_lookup;
+      cost[k] = lookups * lookup_b[k] + static_cast<int64_t>(B) * bag_b[k];
+      traffic += real ? static_cast<float>(cost[k]) : 0.f;
+      one_per_bag = lookups == B && first_lookup == 0;
+    }
+    s.cand[f] = cand[k];
+    if constexpr (BindingStorage<F>::kKeepAddrs) {
+      s.offsets_addr[f] = offs_at[k];
+      s.indices_addr[f] = idx_at[k];
+      s.table_addr[f] = table_at[k];
+      s.one_per_bag[f] = one_per_bag;
+    }
+  }
 
-  // Automatic tile size: bind with the smallest size and add up the batch's traffic on the
-  // way; only a batch large enough for bigger tiles is bound a second time.
+  // Step 2 (only where the tile size or the split unit depend on it): the batch's traffic, in
+  // single precision -- it sizes tiles in steps of kilobytes.
   const bool automatic = tile_bytes <= 0 && !fixed_tiles;
   const bool need_total = automatic || (SPLIT && !fixed_tiles);
-  long long traffic = bind_features(automatic ? kAutoTileMin : tile_bytes, 0);
+  int tile_size = tile_bytes;
+  long long split_unit = 0;
   if (need_total) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) traffic += __shfl_xor(traffic, d, 64);
-    if ((tid & 63) == 0) s.partial[tid >> 6] = traffic;
-  }
-  if (tid == 0) s.prefix[0] = 0;
-  __syncthreads();
-  if (need_total) {
-    long long total = 0;
-    for (int w = 0; w < BT / 64; ++w) total += s.partial[w];
-    int tile_size = tile_bytes;
-    if (automatic) {
-      long long t = total / (static_cast<long long>(grid_blocks) * kAutoTilesPerWorkgroup);
-      t = t < kAutoTileMin ? kAutoTileMin : (t > kAutoTileMax ? kAutoTileMax : t);
-      tile_size = static_cast<int>(t) & ~4095;
+    float total = wave_sum(traffic);
+    if constexpr (!ONE_WAVE) {
+      float *partial = reinterpret_cast<float *>(s.partial);
+      if ((tid & 63) == 0) partial[tid >> 6] = total;
+      __syncthreads();
+      total = 0.f;
+      for (int w = 0; w < BT / 64; ++w) total += partial[w];
     }
-    long long split_unit = 0;
+    const long long total_bytes = static_cast<long long>(total);
+    if (automatic) tile_size = auto_tile_size(total_bytes, grid_blocks);
     if (SPLIT) {
-      split_unit = total / (4ll * (grid_blocks > 0 ? grid_blocks : 1));
+      split_unit = total_bytes / (4ll * (grid_blocks > 0 ? grid_blocks : 1));
       if (split_unit < tile_size) split_unit = tile_size;
       if (split_unit < kSplitMinUnit) split_unit = kSplitMinUnit;
     }
-    // the same decision in every thread of the grid
-    if (SPLIT || tile_size != kAutoTileMin) {
-      bind_features(tile_size, split_unit);
-      __syncthreads();
-    }
   }
-  if (tid < 64) {
-    int carry = 0;
-    for (int c = 0; c < F; c += 64) {
-      const int i = c + tid;
-      int v = i < F ? s.prefix[i + 1] : 0;
-      v = wave_inclusive_scan(v, tid) + carry;
-      if (i < F) s.prefix[i + 1] = v;
-      carry = __shfl(v, 63, 64);
+
+  // Step 3: tiles of every feature, from registers.
+  int tiles_of[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const bool real = tid + k * BT < F;
+    const int f = min(tid + k * BT, F - 1);
+    int g = gran[k];
+    const bool may_split = g == kSplitGran && !fixed_tiles;
+    if (g == kSplitGran) g = 1;
+    const int64_t want = fixed_tiles ? fixed_tiles[f] : approx_ceil_div(cost[k], tile_size);
+    // mean traffic of one bag of this feature
+    const int64_t bag_cost = B > 0 ? static_cast<int64_t>(static_cast<float>(cost[k]) /
+                                                          static_cast<float>(B)) : 0;
+    int tiles = want < 1 ? 1 : (want > B ? B : static_cast<int>(want));
+    int bpt = 0;
+    int64_t parts = 1;
+    if (SPLIT && may_split && B > 0 && split_unit > 0 && bag_cost > 2 * split_unit) {
+      parts = approx_ceil_div(bag_cost, split_unit);
+      if (parts > kBindMaxParts) parts = kBindMaxParts;
+      if (parts * B > kBindMaxSplitTiles) parts = kBindMaxSplitTiles / B;
+    }
+    if (parts > 1) {
+      tiles = B * static_cast<int>(parts);
+      bpt = -static_cast<int>(parts);
+    } else if (B > 0) {
+      bpt = (B + tiles - 1) / tiles;
+      // Tiles are whole workgroup passes (g bags) -- unless one pass of this schedule is more
+      // than kMaxTileFactor times the traffic a tile should carry: then the tile keeps its
+      // share of the traffic and some of the schedule's teams idle.
+      const int whole = (bpt + g - 1) / g * g;
+      if (fixed_tiles || bpt >= g ||
+          static_cast<int64_t>(whole) * bag_cost <= static_cast<int64_t>(kMaxTileFactor) * tile_size)
+        bpt = whole;
+      tiles = (B + bpt - 1) / bpt;
+    } else {
+      tiles = 0;
+    }
+    // (a surplus thread may have sized its tiles from another wavefront's view of the total)
+    if (real) s.bags_per_tile[f] = bpt;
+    tiles_of[k] = real ? tiles : 0;
+  }
+
+  // Step 4: prefix[f] = first tile of feature f.
+  if constexpr (ONE_WAVE) {
+    if (tid < 64) {
+      const int incl = wave_inclusive_scan(tiles_of[0], tid);
+      if (tid < F) s.prefix[tid + 1] = incl;
+      if (tid == 0) s.prefix[0] = 0;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int f = tid + k * BT;
+      if (f < F) s.prefix[f + 1] = tiles_of[k];
+    }
+    if (tid == 0) s.prefix[0] = 0;
+    __syncthreads();
+    if (tid < 64) {
+      int carry = 0;
+      for (int c = 0; c < F; c += 64) {
+        const int i = c + tid;
+        int v = i < F ? s.prefix[i + 1] : 0;
+        v = wave_inclusive_scan(v, tid) + carry;
+        if (i < F) s.prefix[i + 1] = v;
+        carry = __shfl(v, 63, 64);
+      }
     }
   }
   __syncthreads();
@@ -241,6 +374,26 @@ __device__ __forceinline__ int find_feature(const int *prefix, const int tile) {
 template <int F>
 __device__ __forceinline__ int find_feature(const BindingStorage<F> &s, const int tile) {
   return find_feature<F>(s.prefix, tile);
+}
+
+// The same for a whole wavefront at once (`tile` the same in all its lanes; every lane gets the
+// answer): the number of features whose first tile is at or before `tile`, counted 64 features
+// at a time with independent LDS reads and ballots instead of log2(F) dependent ones.
+template <int F>
+__device__ __forceinline__ int find_feature_wave(const int *prefix, const int tile) {
+  if constexpr (F > 512) {
+    return find_feature<F>(prefix, tile);
+  } else {
+    const int lane = threadIdx.x & 63;
+    int count = 0;
+#pragma unroll
+    for (int base = 0; base < F; base += 64) {
+      const int f = base + lane + 1;            // prefix[f] <= tile: feature f starts at or before it
+      const bool at_or_before = f <= F - 1 && prefix[f] <= tile;
+      count += __builtin_popcountll(__builtin_amdgcn_ballot_w64(at_or_before));
+    }
+    return count;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------

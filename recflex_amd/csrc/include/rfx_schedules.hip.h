@@ -456,6 +456,117 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
 }
 
 // ---------------------------------------------------------------------------------------------
+// onehot_bags: bags of at most one lookup (the pooled output row is a copy of a table row, or
+// zeros), X column lanes per bag, no lookup lanes.  Such a feature costs latencies, not
+// arithmetic: offsets -> index -> row -> store is a chain of three round trips to memory per
+// pass, so a wavefront takes UB bags per team at once (64 / X teams: (64 / X) * UB bags and as
+// many row loads in flight per pass) and, when the binding found exactly as many lookups as
+// bags in the batch (one_per_bag), fetches indices[bag] together with the offsets instead of
+// after them -- right whenever offsets[bag] == bag, which is then checked.  A wavefront that
+// meets a longer bag in its pass hands that pass to team_bags.
+//
+// Wavefront w of the workgroup owns the bags [bag_begin + (w + k * BT/64) * WB, + WB), WB =
+// (64 / X) * UB; within it team t takes bags t, t + 64/X, ...: consecutive lanes of an offsets or
+// index load read consecutive words.
+//
+// Reference counterpart: onehot::GatherSegments (examples/csrc/include/onehot_kernel.cuh:14-87),
+// which copies rows with 4-byte accesses and takes the bag length of 1 for granted.
+// ---------------------------------------------------------------------------------------------
+template <int BT, int DT, int D, int X, int UB, int OVEC>
+__device__ __forceinline__ void
+onehot_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
+            const int *__restrict__ indices, const int *__restrict__ offsets,
+            float *__restrict__ out, const int esum, const int col_off, const int bag_begin,
+            const int bag_end, const int skip_longer_than, const int one_per_bag) {
+  using R = Row<DT, D>;
+  static_assert(X >= 1 && X <= 64 && (X & (X - 1)) == 0, "column lanes: a power of two <= 64");
+  constexpr int TEAMS_W = 64 / X;               // teams per wavefront
+  constexpr int WB = TEAMS_W * UB;              // bags per wavefront and pass
+  constexpr int WAVES = BT / 64;
+  constexpr int VPL = ceil_div(R::V, X);
+  constexpr int VB = R::VB;
+  constexpr int EPV = R::EPV;
+
+  const int tid = body_thread_id<BT>();
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int team = lane / X;
+  const int x = lane - team * X;
+
+  for (int pass0 = bag_begin + wave * WB; pass0 < bag_end; pass0 += WAVES * WB) {
+    const int pass_end = min(pass0 + WB, bag_end);
+    int bag[UB], beg[UB], len[UB], spec[UB];
+    // first round trip: the bags' bounds, and on the hint the index each would have
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      bag[u] = pass0 + u * TEAMS_W + team;
+      const int b = min(bag[u], bag_end - 1);
+      beg[u] = offsets[b];
+      len[u] = bag[u] < pass_end ? offsets[b + 1] - beg[u] : 0;
+      spec[u] = one_per_bag ? indices[b] : 0;   // exactly `batch` lookups exist: in bounds
+    }
+    bool mine = true;         // every bag of this lane has zero or one lookup
+    bool guessed = true;      // ... and the one lookup is where the hint says
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      mine = mine && len[u] <= 1;
+      guessed = guessed && (len[u] == 0 || beg[u] == bag[u]);
+    }
+    if (__builtin_amdgcn_ballot_w64(!mine) != 0) {
+      // the general routine for this wavefront's bags (it also knows what to do with very long ones)
+      team_bags<64, DT, D, X, 1, 2, 1, VPL, OVEC>(
+          stage ? stage + wave * (64 * kStageF4PerLane) : nullptr, table, indices, offsets, out,
+          esum, col_off, pass0, pass_end, skip_longer_than);
+      continue;
+    }
+    int idx[UB];
+    if (one_per_bag && __builtin_amdgcn_ballot_w64(!guessed) == 0) {
+#pragma unroll
+      for (int u = 0; u < UB; ++u) idx[u] = len[u] == 1 ? spec[u] : -1;
+    } else {
+#pragma unroll
+      for (int u = 0; u < UB; ++u) idx[u] = len[u] == 1 ? indices[beg[u]] : -1;
+    }
+    // the rows
+    Vec<VB> buf[UB][VPL];
+    f32x2 sb[UB];
+#pragma unroll
+    for (int u = 0; u < UB; ++u)
+      if (idx[u] >= 0) {
+        const char *row = table + static_cast<int64_t>(idx[u]) * R::STRIDE;
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+          const int c = x + v * X;
+          if (c < R::V) buf[u][v] = load_vec<VB>(row + c * VB);
+        }
+        if constexpr (DT == I8) sb[u] = load_scale_bias<D>(row);
+      }
+    // 0 + row, as the sum of a bag of one lookup is formed everywhere else (an empty bag: zeros)
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      if (bag[u] >= pass_end) continue;
+      float *dst = out + static_cast<int64_t>(bag[u]) * esum + col_off;
+#pragma unroll
+      for (int v = 0; v < VPL; ++v) {
+        const int c = x + v * X;
+        if (c >= R::V) continue;
+        float acc[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) acc[e] = 0.f;
+        if (idx[u] >= 0) {
+          accumulate<DT, VB>(acc, buf[u][v], DT == I8 ? sb[u].x : 1.f);
+          if constexpr (DT == I8) {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) acc[e] += sb[u].y;
+          }
+        }
+        store_floats<EPV, OVEC>(dst + c * EPV, acc);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // block_bags: the whole workgroup sums one bag at a time (long bags).  The bag's indices are
 // staged in LDS in chunks of CHUNK with coalesced loads; lane (y, x) reads index y + k*Y of the
 // chunk and vector(s) x of the row; the Y lookup lanes inside a wavefront are combined with the

@@ -1,0 +1,139 @@
+"""HBM traffic per launch of the prebuilt libraries, as hardware counters gave it.
+
+A live benchmark run cannot read the memory counters; ``rocprofv3 --pmc FETCH_SIZE`` and
+``--pmc WRITE_SIZE`` runs of ``bench.py`` can.  This module turns the two counter files of such
+runs into one record per model in ``recflex_amd/tuned/hbm_traffic.json`` and hands the figure
+back to ``bench.py`` -- but only for the very library it was measured on: every record carries a
+key over the model's emitted source and the device headers, and a library built from anything
+else gets ``None``.
+
+    python -m recflex_amd.hbm_traffic record --model c3_tuned \\
+        --fetch-csv gpurun_out/pmc_fetch_c3/x_counter_collection.csv \\
+        --write-csv gpurun_out/pmc_write_c3/x_counter_collection.csv --copy-bytes 805306368
+
+``FETCH_SIZE`` / ``WRITE_SIZE`` are what the L2 caches exchange with the memory side, in units
+that a plain copy of known size calibrates: the runs hold one device-to-device copy of
+``--copy-bytes`` bytes (``bench.py --copy-calibration``), and each counter is scaled by
+bytes copied / counter reading of that copy.
+"""
+
+import argparse
+import csv
+import glob
+import hashlib
+import json
+import os
+from typing import Dict, List, Optional, Tuple
+
+from .code_emitter.build_basic import BasicBuilder
+from . import prebuilt
+
+RECORD_PATH = os.path.join(prebuilt.TUNED_DIR, "hbm_traffic.json")
+
+
+def library_key(model: str) -> Optional[str]:
+    """Key of what the model's library is built from: its emitted ``process.hip`` and the device
+    headers.  ``None`` if the model was never emitted here."""
+    src = os.path.join(prebuilt.model_dir(model), "process.hip")
+    if not os.path.exists(src):
+        return None
+    h = hashlib.sha256()
+    for path in [src] + BasicBuilder().device_headers():
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:24]
+
+
+def load_records() -> Dict[str, dict]:
+    if not os.path.exists(RECORD_PATH):
+        return {}
+    with open(RECORD_PATH) as f:
+        return json.load(f)
+
+
+def recorded_traffic_bytes(model: str) -> Optional[float]:
+    """HBM bytes per launch of ``FusedKnl`` of this model, if counters were taken on the library
+    as it is built now; ``None`` otherwise."""
+    rec = load_records().get(model)
+    if not rec or rec.get("key") != library_key(model):
+        return None
+    return float(rec["bytes"])
+
+
+def _counter_files(path: str) -> List[str]:
+    if os.path.isfile(path):
+        return [path]
+    return sorted(glob.glob(os.path.join(path, "**", "*counter_collection.csv"), recursive=True))
+
+
+def read_counter(path: str, counter: str) -> Dict[str, List[float]]:
+    """kernel name -> value of ``counter`` per dispatch, from rocprofv3 ``--pmc`` csv output."""
+    out: Dict[str, List[float]] = {}
+    for fname in _counter_files(path):
+        with open(fname, newline="") as f:
+            for row in csv.DictReader(f):
+                if row.get("Counter_Name") == counter:
+                    out.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+    if not out:
+        raise ValueError(f"no {counter} readings under {path}")
+    return out
+
+
+def _fused_and_copy(readings: Dict[str, List[float]], copy_substr: str) -> Tuple[float, int, float]:
+    """(mean reading of FusedKnl, its dispatches, largest reading of a copy kernel)."""
+    fused = readings.get("FusedKnl")
+    if not fused:
+        raise ValueError("the counter file holds no FusedKnl dispatch")
+    copies = [v for name, vals in readings.items() if copy_substr in name for v in vals]
+    if not copies:
+        raise ValueError(f"the counter file holds no kernel named *{copy_substr}* to calibrate with")
+    return sum(fused) / len(fused), len(fused), max(copies)
+
+
+def record(model: str, fetch_csv: str, write_csv: str, copy_bytes: int,
+           copy_substr: str = "copyBuffer") -> dict:
+    key = library_key(model)
+    if key is None:
+        raise FileNotFoundError(f"{prebuilt.model_dir(model)}/process.hip: build the model first")
+    fetch, n_fetch, copy_fetch = _fused_and_copy(read_counter(fetch_csv, "FETCH_SIZE"), copy_substr)
+    write, n_write, copy_write = _fused_and_copy(read_counter(write_csv, "WRITE_SIZE"), copy_substr)
+    fetch_factor = copy_bytes / copy_fetch          # bytes per counter unit
+    write_factor = copy_bytes / copy_write
+    rec = {
+        "key": key,
+        "fetch_reading": fetch, "write_reading": write,
+        "fetch_bytes_per_unit": fetch_factor, "write_bytes_per_unit": write_factor,
+        "read_bytes": fetch * fetch_factor, "written_bytes": write * write_factor,
+        "bytes": fetch * fetch_factor + write * write_factor,
+        "dispatches": [n_fetch, n_write],
+        "calibration": f"largest *{copy_substr}* dispatch = a copy of {copy_bytes} bytes",
+    }
+    records = load_records()
+    records[model] = rec
+    with open(RECORD_PATH, "w") as f:
+        json.dump(records, f, indent=1, sort_keys=True)
+    return rec
+
+
+def main() -> None:
+    parser = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    sub = parser.add_subparsers(dest="cmd", required=True)
+    rec = sub.add_parser("record", help="turn a FETCH_SIZE and a WRITE_SIZE run into a record")
+    rec.add_argument("--model", required=True, help="prebuilt model name, e.g. c3_tuned")
+    rec.add_argument("--fetch-csv", required=True)
+    rec.add_argument("--write-csv", required=True)
+    rec.add_argument("--copy-bytes", type=int, required=True)
+    rec.add_argument("--copy-kernel", default="copyBuffer", help="substring of the copy kernel's name")
+    sub.add_parser("show", help="print the records and whether each matches the library as built now")
+    args = parser.parse_args()
+    if args.cmd == "record":
+        print(json.dumps(record(args.model, args.fetch_csv, args.write_csv, args.copy_bytes,
+                                args.copy_kernel), indent=1))
+    else:
+        for model, r in load_records().items():
+            print(f"{model}: {r['bytes'] / 1e6:.1f} MB per launch "
+                  f"({'current' if r['key'] == library_key(model) else 'STALE: library changed'})")
+
+
+if __name__ == "__main__":
+    main()

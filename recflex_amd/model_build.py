@@ -53,8 +53,11 @@ def build_model(output_dir: str, feat_schedules: FeatSchedules, rebuild: bool = 
 
 
 def default_feat_schedules(metas: Sequence[MetaData], mean_bag_lens: Sequence[float],
-                           block_threads: int = 256) -> FeatSchedules:
-    return [default_schedule(m, l, block_threads) for m, l in zip(metas, mean_bag_lens)]
+                           block_threads: int = 256, one_hot: Sequence[bool] = None) -> FeatSchedules:
+    """``one_hot[f]``: no bag of feature ``f`` holds more than one lookup, as far as is known."""
+    one_hot = one_hot or [False] * len(metas)
+    return [default_schedule(m, l, block_threads, one_hot=h)
+            for m, l, h in zip(metas, mean_bag_lens, one_hot)]
 
 
 def load_feat_schedules(schedule_json: str, block_threads: int = 256) -> FeatSchedules:

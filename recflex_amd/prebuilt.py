@@ -69,8 +69,13 @@ def expected_bag_len(f: FeatureSpec) -> float:
 DEFAULT_OCCUPANCY = 4
 
 
+def is_one_hot(f: FeatureSpec) -> bool:
+    return f.fixed_len and round(f.mean_bag) <= 1
+
+
 def _default(wl: Workload, occupancy: Optional[int] = DEFAULT_OCCUPANCY, **emit_kwargs) -> ModelSpec:
-    fs = default_feat_schedules(metas_of(wl), [expected_bag_len(f) for f in wl.features], BLOCK_THREADS)
+    fs = default_feat_schedules(metas_of(wl), [expected_bag_len(f) for f in wl.features], BLOCK_THREADS,
+                                one_hot=[is_one_hot(f) for f in wl.features])
     return ModelSpec(wl, fs, occupancy, emit_kwargs)
 
 

@@ -10,7 +10,8 @@ from typing import Dict, NamedTuple, Tuple, Type
 from recflex_amd.code_emitter.schedule_base import ScheduleBase, MetaData
 from .team import (TeamParams, TeamScheduleBase, ThreadPerBagSchedule, ThreadPerBagParams,
                    SubWavefrontPerBagSchedule, SubWavefrontPerBagParams,
-                   WavefrontPerBagSchedule, WavefrontPerBagParams, next_pow2)
+                   WavefrontPerBagSchedule, WavefrontPerBagParams, OneHotBagSchedule,
+                   OneHotBagParams, next_pow2)
 from .block_per_bag import BlockPerBagSchedule, BlockPerBagParams, SplitBagSchedule
 from .reference_names import (OneHotSchedule, OneHotMultiBlockSchedule, WarpPerSampleSchedule,
                               OneBlockMultiSampleSchedule, MultiBlockPerSampleSchedule,
@@ -21,7 +22,7 @@ from .reference_names import (OneHotSchedule, OneHotMultiBlockSchedule, WarpPerS
 SCHEDULE_MAPPING: Dict[str, Type[ScheduleBase]] = {
     cls.__name__: cls
     for cls in (ThreadPerBagSchedule, SubWavefrontPerBagSchedule, WavefrontPerBagSchedule,
-                BlockPerBagSchedule, SplitBagSchedule, OneHotSchedule, OneHotMultiBlockSchedule,
+                OneHotBagSchedule, BlockPerBagSchedule, SplitBagSchedule, OneHotSchedule, OneHotMultiBlockSchedule,
                 WarpPerSampleSchedule, OneBlockMultiSampleSchedule,
                 MultiBlockPerSampleSchedule, ReduceByKeySchedule)
 }
@@ -32,8 +33,9 @@ PARAM_TYPES: Dict[str, Type[NamedTuple]] = {
     "WavefrontPerBagSchedule": WavefrontPerBagParams,
     "BlockPerBagSchedule": BlockPerBagParams,
     "SplitBagSchedule": BlockPerBagParams,
-    "OneHotSchedule": TeamParams,
-    "OneHotMultiBlockSchedule": TeamParams,
+    "OneHotBagSchedule": OneHotBagParams,
+    "OneHotSchedule": OneHotBagParams,
+    "OneHotMultiBlockSchedule": OneHotBagParams,
     "WarpPerSampleSchedule": TeamParams,
     "OneBlockMultiSampleSchedule": TeamParams,
     "MultiBlockPerSampleSchedule": BlockPerBagParams,
@@ -41,14 +43,19 @@ PARAM_TYPES: Dict[str, Type[NamedTuple]] = {
 }
 
 
-def default_schedule(meta: MetaData, mean_bag_len: float = 1.0,
-                     block_threads: int = 256) -> Tuple[ScheduleBase, NamedTuple]:
-    """Untuned starting point for one feature from its row size and mean bag length: enough
+def default_schedule(meta: MetaData, mean_bag_len: float = 1.0, block_threads: int = 256,
+                     one_hot: bool = False) -> Tuple[ScheduleBase, NamedTuple]:
+    """Untuned starting point for one feature from its row size and mean bag length
+    (``one_hot``: no bag of the feature is known to hold more than one lookup -- the row-copy
+    template): enough
     column lanes that a lane owns one or two 16-byte vectors, lookup lanes only for long bags,
     and two to four independent row loads in flight per lane -- fewer for fp16 and int8 rows,
     whose 8 or 16 fp32 accumulators per 16-byte vector would otherwise push the fused kernel past
     the registers that four or five workgroups per CU leave it (measured on C4 and C5: 2 % and
     17 % faster than with four loads in flight everywhere)."""
+    if one_hot:
+        sched = OneHotBagSchedule(meta, block_threads)
+        return sched, sched.default_params()
     v = meta.row_vectors
     x = min(64, next_pow2(v))
     if v > 1 and x * meta.vec_bytes >= 256 and mean_bag_len < 8:

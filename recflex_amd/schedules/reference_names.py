@@ -5,7 +5,8 @@ Each name keeps the role it has in the reference and draws its candidates from t
 templates:
 
 =============================  ==========================================================
-``OneHotSchedule``             bags of one lookup: no lookup lanes, several bags in flight
+``OneHotSchedule``             bags of one lookup: the row-copy template (``OneHotBagSchedule``),
+                               no lookup lanes, several bags in flight per team
 ``OneHotMultiBlockSchedule``   same (the reference variant differs only in its block count,
                                which the run-time binding decides here)
 ``WarpPerSampleSchedule``      X column lanes, serial lookups, no cross-lane reduction
@@ -20,7 +21,7 @@ from typing import List
 
 from recflex_amd.code_emitter.schedule_base import InputStats
 from .team import (TeamScheduleBase, TeamParams, fits_registers, next_pow2, _pow2_upto,
-                   passes_for, MAX_ACC_FLOATS)
+                   passes_for, MAX_ACC_FLOATS, OneHotBagSchedule, OneHotBagParams)
 from .block_per_bag import SplitBagSchedule, BlockPerBagParams
 
 
@@ -33,22 +34,11 @@ class _GenericTeam(TeamScheduleBase):
         return TeamParams(*params)
 
 
-class OneHotSchedule(_GenericTeam):
-    def GenParamCandidates(self, stats: InputStats = None) -> List[TeamParams]:
-        m = self.meta
-        out = []
-        for x in _pow2_upto(min(64, next_pow2(m.row_vectors))):
-            vpl = -(-m.row_vectors // x)
-            if vpl > 16:
-                continue
-            for bags in (1, 2, 4, 8):
-                p = TeamParams(x, 1, 1, bags, _vpp(m, vpl))
-                if fits_registers(m, p):
-                    out.append(p)
-        return out
+class OneHotSchedule(OneHotBagSchedule):
+    pass
 
 
-class OneHotMultiBlockSchedule(OneHotSchedule):
+class OneHotMultiBlockSchedule(OneHotBagSchedule):
     pass
 
 
@@ -94,8 +84,8 @@ class ReduceByKeySchedule(SplitBagSchedule):
 
 
 # parameter tuple names of the reference, for scripts that import them
-OneHotParams = TeamParams
-OneHotMultiBlockParams = TeamParams
+OneHotParams = OneHotBagParams
+OneHotMultiBlockParams = OneHotBagParams
 WarpPerSampleParams = TeamParams
 OneBlockMultiSampleParams = TeamParams
 MultiBlockPerSampleParams = BlockPerBagParams

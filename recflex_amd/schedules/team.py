@@ -201,3 +201,80 @@ class WavefrontPerBagSchedule(TeamScheduleBase):
                 if fits_registers(m, self.team_params(p)):
                     out.append(p)
         return out
+
+
+class OneHotBagParams(NamedTuple):
+    lanes_x: int
+    bags_per_team: int
+
+
+class OneHotBagSchedule(ScheduleBase):
+    """Bags of at most one lookup: ``rfx::onehot_bags``, X column lanes per bag, ``bags_per_team``
+    bags (and row loads) in flight per team, the index fetched together with the bag's offsets
+    when the batch holds exactly one lookup per bag.  A wavefront whose pass holds a longer bag
+    runs that pass through ``rfx::team_bags``, so the schedule is right for any input and fast
+    for the input it is meant for.
+
+    Reference counterpart: ``OneHotSchedule`` / ``OneHotMultiBlockSchedule``
+    (examples/schedules/one_hot.py:22-92, one_hot_multi_block.py), whose kernel takes the bag
+    length of 1 for granted."""
+
+    # row vectors a lane holds in flight at most (bags_per_team x vectors per lane)
+    MAX_VECTORS_IN_FLIGHT = 16
+
+    def _check(self, p: OneHotBagParams) -> None:
+        x = p.lanes_x
+        if x < 1 or x > 64 or x & (x - 1):
+            raise ValueError(f"lanes_x={x} is not a power of two <= 64")
+        if self.block_threads % 64:
+            raise ValueError(f"block_threads={self.block_threads} must hold whole wavefronts")
+        if p.bags_per_team < 1:
+            raise ValueError("bags_per_team must be >= 1")
+
+    def EmitScheduleBody(self, params: OneHotBagParams) -> str:
+        self._check(params)
+        v = self.sched_vars
+        m = self.meta
+        return f'''
+  rfx::onehot_bags<{v.BLOCK_THREADS}, {m.dtype_id}, {m.embed_dim}, {params.lanes_x},
+                   {params.bags_per_team}, {v.out_vec}>(
+      {v.stage},
+      {v.embed_table}, {v.indices}, {v.offsets}, {v.output},
+      {v.out_row_stride}, {v.embed_dim_offset}, {v.bag_begin}, {v.bag_end}, {v.skip_long},
+      {v.one_per_bag});
+'''
+
+    def EmitShmemType(self, params: OneHotBagParams) -> str:
+        return "char"
+
+    def NeedsOutputStage(self, params: OneHotBagParams) -> bool:
+        # the general routine behind it stages fp16 / int8 outputs through LDS
+        return self.meta.elems_per_vector > 4
+
+    def LongBagThreshold(self, params: OneHotBagParams) -> int:
+        return 64           # rfx::long_bag_threshold(2, 1) of the general routine behind it
+
+    def TileGranularity(self, params: OneHotBagParams) -> int:
+        return self.block_threads // params.lanes_x * params.bags_per_team
+
+    def GenParamCandidates(self, stats: InputStats = None) -> List[OneHotBagParams]:
+        m = self.meta
+        out = []
+        for x in _pow2_upto(min(64, next_pow2(m.row_vectors))):
+            vpl = -(-m.row_vectors // x)
+            if vpl > 8:
+                continue
+            for bags in (1, 2, 4, 8):
+                if bags * vpl <= self.MAX_VECTORS_IN_FLIGHT:
+                    out.append(OneHotBagParams(x, bags))
+        return out
+
+    def default_params(self) -> OneHotBagParams:
+        """Two row vectors per lane where the row has four or more, two bags per team: four row
+        loads in flight per lane (measured on 26 features x 4 096 bags of 256-byte rows: 8 lanes
+        x 2 bags 8.2 us, 8 x 4 8.7 us, 16 lanes x 2, 4 or 8 bags 12 us and more)."""
+        v = self.meta.row_vectors
+        x = min(64, next_pow2(v))
+        if v >= 4:
+            x //= 2
+        return OneHotBagParams(x, 2)

@@ -434,19 +434,26 @@ class KernelTimer:
 MAX_TILE_FACTOR = 8      # rfx::kMaxTileFactor
 AUTO_TILES_PER_WORKGROUP = 64                       # rfx::kAutoTilesPerWorkgroup
 AUTO_TILE_MIN, AUTO_TILE_MAX = 64 * 1024, 256 * 1024    # rfx::kAutoTileMin / kAutoTileMax
+AUTO_TILE_FLOOR = 4 * 1024                              # rfx::kAutoTileFloor
 
 
 def auto_tile_bytes(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int],
                     bag_bytes: Sequence[int], grid_blocks: int) -> int:
-    """Host restatement of the tile size the device picks when none is given: the batch's
-    traffic over 64 tiles per workgroup of the grid, within 64..256 KiB, in steps of 4 KiB."""
+    """Host restatement of the tile size the device picks when none is given
+    (``rfx::auto_tile_size``): the batch's traffic over 64 tiles per workgroup of the grid, within
+    64..256 KiB, in steps of 4 KiB; a batch of less than 64 KiB per workgroup gets about two tiles
+    per workgroup, at least 4 KiB, in steps of 1 KiB."""
     total = 0
     for off, lb, bb in zip(offsets, lookup_bytes, bag_bytes):
         batch = len(off) - 1
         if batch > 0:
             total += int(off[-1] - off[0]) * lb + batch * bb
-    t = total // (max(1, grid_blocks) * AUTO_TILES_PER_WORKGROUP)
-    return min(max(t, AUTO_TILE_MIN), AUTO_TILE_MAX) & ~4095
+    grid = max(1, grid_blocks)
+    t = total // (grid * AUTO_TILES_PER_WORKGROUP)
+    if t >= AUTO_TILE_MIN:
+        return min(t, AUTO_TILE_MAX) & ~4095
+    t = total // (2 * grid)
+    return min(max(t, AUTO_TILE_FLOOR), AUTO_TILE_MIN) & ~1023
 
 
 def tiles_per_feature(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int],

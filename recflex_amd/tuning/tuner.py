@@ -188,7 +188,7 @@ class Tuner:
                 from recflex_amd.schedules import default_schedule
                 lens = [len(i) / max(1, len(o) - 1) for i, o in self.batches[feat_id]]
                 sched, params = default_schedule(self.metas[feat_id], float(np.mean(lens)) if lens else 1.0,
-                                                 self.basic.block_threads)
+                                                 self.basic.block_threads, one_hot=self.is_one_hot(feat_id))
                 print(f"feature {feat_id}: its schedule classes "
                       f"({', '.join(type(s).__name__ for s in self.feat_schedules[feat_id])}) have no "
                       f"candidate for dim {self.metas[feat_id].embed_dim} {self.metas[feat_id].data_type}; "
@@ -445,6 +445,13 @@ class Tuner:
         with open(path) as f:
             return json.load(f)
 
+    def is_one_hot(self, feat_id: int) -> bool:
+        """No bag of the feature holds more than one lookup in any sampled batch (and there is
+        at least one lookup)."""
+        feat = self.batches[feat_id]
+        longest = max((int(np.diff(off).max()) for _, off in feat if len(off) > 1), default=0)
+        return longest == 1
+
     def default_choices(self) -> List[List[int]]:
         """Index, in every feature's candidate list, of the schedule ``default_schedule`` would
         pick from the mean bag length of the sampled batches (nearest candidate of the same
@@ -455,7 +462,7 @@ class Tuner:
         for feat_id, cands in enumerate(self.feat_sched_param_candidates):
             lens = [len(i) / max(1, len(o) - 1) for i, o in self.batches[feat_id]]
             sched, params = default_schedule(self.metas[feat_id], float(np.mean(lens)),
-                                             self.basic.block_threads)
+                                             self.basic.block_threads, one_hot=self.is_one_hot(feat_id))
             body = sched.EmitScheduleBody(params)
             pick, best_d = 0, None
             for k, (s, p) in enumerate(cands):

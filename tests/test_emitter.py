@@ -212,7 +212,7 @@ def test_split_bag_schedules_get_workspace_regions():
     assert regions == [-1, 0, -1, 2048 * 65] and total == 2048 * (65 + 129)
     src = em.emit_kernel(occupancy=4)
     assert f"SPLIT_BYTES = {total * 4}LL" in src and "c_split_region[feat_idx]" in src
-    assert "rfx::split_bags<" in src and "bind_tiles<NUM_FEATS, BLOCK_THREADS, HAS_SPLIT>" in src
+    assert "rfx::split_bags<" in src and "bind_tiles<NUM_FEATS, BLOCK_THREADS, HAS_SPLIT," in src
     m = re.search(r"c_cand_gran\[\] = \{\s*([-\d,\s]+)\}", src)
     gran = [int(v) for v in m.group(1).split(",")]
     assert gran[1] == -1 and gran[3] == -1 and gran[0] > 0 and gran[2] > 0

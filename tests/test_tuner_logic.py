@@ -293,11 +293,19 @@ def test_profiler_command_uses_absolute_paths(tmp_path, monkeypatch):
 
 def test_automatic_tile_size_rule():
     """The tile size the device chooses when none is given, restated on the host: 64 tiles per
-    workgroup of the grid, clamped to 64..256 KiB, multiples of 4 KiB."""
+    workgroup of the grid, clamped to 64..256 KiB, multiples of 4 KiB; a batch of less than
+    64 KiB per workgroup: two tiles per workgroup, 4..64 KiB, multiples of 1 KiB."""
     from recflex_amd.tuning.measure import auto_tile_bytes
     off = lambda n_bags, per_bag: np.arange(n_bags + 1, dtype=np.int64) * per_bag
-    # tiny batch: the lower bound
-    assert auto_tile_bytes([off(512, 4)] * 4, [132] * 4, [132] * 4, 1024) == 64 * 1024
+    # tiny batch (1.35 MB over 1024 workgroups): the floor
+    assert auto_tile_bytes([off(512, 4)] * 4, [132] * 4, [132] * 4, 1024) == 4 * 1024
+    # 55 MB over 1024 workgroups: half a workgroup's share, 26 KiB
+    total = 26 * (4096 * 260 + 4096 * 260)
+    got = auto_tile_bytes([off(4096, 1)] * 26, [260] * 26, [260] * 26, 1024)
+    assert got == (total // 2048) & ~1023 == 26 * 1024
+    # 3.4 GB over 1024 workgroups: less than 64 KiB per tile at 64 tiles per workgroup, far more
+    # at two -- the lower bound of large batches
+    assert auto_tile_bytes([off(8192, 30)] * 100, [132] * 100, [132] * 100, 1024) == 64 * 1024
     # 10.5 GB over 1280 workgroups: 128 KiB after rounding down to 4 KiB
     got = auto_tile_bytes([off(16384, 20)] * 200, [148] * 200, [516] * 200, 1280)
     total = 200 * (16384 * 20 * 148 + 16384 * 516)
@@ -305,7 +313,7 @@ def test_automatic_tile_size_rule():
     # tens of GB: the upper bound
     assert auto_tile_bytes([off(8192, 300)] * 400, [516] * 400, [516] * 400, 1024) == 256 * 1024
     # a grid of one workgroup and an empty batch do not divide by zero
-    assert auto_tile_bytes([np.zeros(1, dtype=np.int64)], [36], [36], 0) == 64 * 1024
+    assert auto_tile_bytes([np.zeros(1, dtype=np.int64)], [36], [36], 0) == 4 * 1024
 
 
 def test_outlier_tiles_are_switched_on_by_the_sampled_data():
