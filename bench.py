@@ -293,14 +293,8 @@ def main():
         sys.exit(3)
 
     if args.copy_calibration > 0:
-        n = args.copy_calibration // 4
-        src = torch.ones(n, dtype=torch.float32, device="cuda:0")
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        dst.copy_(src)             # reads n*4 bytes, writes n*4 bytes
-        torch.cuda.synchronize()
-        del src, dst
-        torch.cuda.empty_cache()
+        from recflex_amd.gather_probe import calibration_copy
+        calibration_copy(args.copy_calibration)     # reads that many bytes, writes as many
 
     floor = not args.no_gather_floor
     head = run_config(args.workload, args.steps, args.warmup, not args.no_cpu, args.tile_bytes,

@@ -99,7 +99,31 @@ gather_probe_knl(const Chunk *__restrict__ chunks, const int n_chunks, const int
   if (acc.x + acc.y + acc.z + acc.w == 1.2345e38f) sink[threadIdx.x] = acc.x;
 }
 
+// Plain copy of n 16-byte vectors, grid-stride.  Its HBM traffic is known (n * 16 bytes read,
+// n * 16 written), so a counter run that holds one launch of it yields the bytes one unit of a
+// memory counter stands for.  The name is unique on purpose: a counter file is searched for it.
+__global__ void __launch_bounds__(256)
+CalibrationCopyKnl(const f32x4 *__restrict__ src, f32x4 *__restrict__ dst, const int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
+    dst[i] = src[i];
+}
+
 } // namespace
+
+// Copies `bytes` (a multiple of 16; both pointers 16-byte aligned, buffers disjoint) from src to
+// dst on `stream` with CalibrationCopyKnl.  Returns the hipError_t of the launch.
+extern "C" int calibration_copy_launch(const void *src, void *dst, int64_t bytes, int grid_blocks,
+                                       void *stream) {
+  if (!src || !dst || bytes < 0 || bytes % 16 != 0 || grid_blocks <= 0 ||
+      reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0)
+    return static_cast<int>(hipErrorInvalidValue);
+  if (bytes == 0) return 0;
+  hipLaunchKernelGGL(CalibrationCopyKnl, dim3(grid_blocks), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const f32x4 *>(src),
+                     static_cast<f32x4 *>(dst), bytes / 16);
+  return static_cast<int>(hipGetLastError());
+}
 
 // Launches the probe on `stream` (asynchronous).  chunks: device array of n_chunks records
 // {int32 feat, begin, count, log2x}; table_ptrs / index_ptrs: device int64[F]; row_strides /

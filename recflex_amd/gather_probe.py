@@ -52,6 +52,36 @@ def make_chunks(num_lookups: Sequence[int], row_vectors: Sequence[int],
     return np.asarray(out, dtype=np.int32).reshape(-1, 4)
 
 
+CALIBRATION_KERNEL = "CalibrationCopyKnl"
+
+
+def calibration_copy(nbytes: int, device="cuda:0") -> None:
+    """One launch of ``CalibrationCopyKnl`` copying ``nbytes`` (rounded down to 16) between two
+    fresh device buffers: the dispatch of known traffic that a memory-counter run is scaled by."""
+    import torch
+    path = lib_path()
+    if not os.path.exists(path):
+        raise FileNotFoundError(f"{path} is missing: build it with recflex_amd.gather_probe.build()")
+    lib = ctypes.CDLL(path)
+    lib.calibration_copy_launch.restype = ctypes.c_int
+    lib.calibration_copy_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+                                            ctypes.c_int, ctypes.c_void_p]
+    n = nbytes // 16 * 4
+    src = torch.ones(n, dtype=torch.float32, device=device)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    blocks = torch.cuda.get_device_properties(device).multi_processor_count * 8
+    rc = lib.calibration_copy_launch(src.data_ptr(), dst.data_ptr(), n * 4, blocks,
+                                     torch.cuda.current_stream(device).cuda_stream)
+    if rc:
+        raise RuntimeError(f"calibration_copy_launch: hipError_t {rc}")
+    torch.cuda.synchronize()
+    if not bool((dst[:: max(1, n // 1024)] == 1).all()):
+        raise RuntimeError("calibration copy: destination differs from source")
+    del src, dst
+    torch.cuda.empty_cache()
+
+
 class GatherProbe:
     def __init__(self, device, tables, d_indices, row_strides: Sequence[int]):
         import torch

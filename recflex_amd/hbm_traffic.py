@@ -13,8 +13,9 @@ else gets ``None``.
 
 ``FETCH_SIZE`` / ``WRITE_SIZE`` are what the L2 caches exchange with the memory side, in units
 that a plain copy of known size calibrates: the runs hold one device-to-device copy of
-``--copy-bytes`` bytes (``bench.py --copy-calibration``), and each counter is scaled by
-bytes copied / counter reading of that copy.
+``--copy-bytes`` bytes by a kernel of a name no library shares, ``CalibrationCopyKnl``
+(``bench.py --copy-calibration``), and each counter is scaled by bytes copied / counter reading
+of that dispatch.
 """
 
 import argparse
@@ -27,6 +28,8 @@ from typing import Dict, List, Optional, Tuple
 
 from .code_emitter.build_basic import BasicBuilder
 from . import prebuilt
+
+CALIBRATION_KERNEL = "CalibrationCopyKnl"      # launched by gather_probe.calibration_copy
 
 RECORD_PATH = os.path.join(prebuilt.TUNED_DIR, "hbm_traffic.json")
 
@@ -80,18 +83,20 @@ def read_counter(path: str, counter: str) -> Dict[str, List[float]]:
 
 
 def _fused_and_copy(readings: Dict[str, List[float]], copy_substr: str) -> Tuple[float, int, float]:
-    """(mean reading of FusedKnl, its dispatches, largest reading of a copy kernel)."""
+    """(mean reading of FusedKnl, its dispatches, reading of the one calibration copy)."""
     fused = readings.get("FusedKnl")
     if not fused:
         raise ValueError("the counter file holds no FusedKnl dispatch")
     copies = [v for name, vals in readings.items() if copy_substr in name for v in vals]
     if not copies:
         raise ValueError(f"the counter file holds no kernel named *{copy_substr}* to calibrate with")
-    return sum(fused) / len(fused), len(fused), max(copies)
+    if len(copies) != 1:
+        raise ValueError(f"{len(copies)} dispatches named *{copy_substr}*: the calibration needs exactly one")
+    return sum(fused) / len(fused), len(fused), copies[0]
 
 
 def record(model: str, fetch_csv: str, write_csv: str, copy_bytes: int,
-           copy_substr: str = "copyBuffer") -> dict:
+           copy_substr: str = CALIBRATION_KERNEL) -> dict:
     key = library_key(model)
     if key is None:
         raise FileNotFoundError(f"{prebuilt.model_dir(model)}/process.hip: build the model first")
@@ -106,7 +111,7 @@ def record(model: str, fetch_csv: str, write_csv: str, copy_bytes: int,
         "read_bytes": fetch * fetch_factor, "written_bytes": write * write_factor,
         "bytes": fetch * fetch_factor + write * write_factor,
         "dispatches": [n_fetch, n_write],
-        "calibration": f"largest *{copy_substr}* dispatch = a copy of {copy_bytes} bytes",
+        "calibration": f"the {copy_substr} dispatch = a copy of {copy_bytes} bytes",
     }
     records = load_records()
     records[model] = rec
@@ -123,7 +128,7 @@ def main() -> None:
     rec.add_argument("--fetch-csv", required=True)
     rec.add_argument("--write-csv", required=True)
     rec.add_argument("--copy-bytes", type=int, required=True)
-    rec.add_argument("--copy-kernel", default="copyBuffer", help="substring of the copy kernel's name")
+    rec.add_argument("--copy-kernel", default=CALIBRATION_KERNEL, help="substring of the copy kernel's name")
     sub.add_parser("show", help="print the records and whether each matches the library as built now")
     args = parser.parse_args()
     if args.cmd == "record":

@@ -254,8 +254,23 @@ class Tuner:
     # ---- compile cache: identical device sources are built once -----------------------------
 
     def _source_key(self, output_dir: str) -> str:
+        """Key of everything a library is compiled from: the emitted source and the device
+        headers it includes (a header edited between two runs must not find the old build)."""
+        h = hashlib.sha256()
         with open(f"{output_dir}/process.hip", "rb") as f:
-            return hashlib.sha256(f.read()).hexdigest()[:24]
+            h.update(f.read())
+        h.update(self._headers_digest())
+        return h.hexdigest()[:24]
+
+    def _headers_digest(self) -> bytes:
+        if not hasattr(self, "_headers_digest_cache"):
+            from recflex_amd.code_emitter.build_basic import BasicBuilder
+            h = hashlib.sha256()
+            for path in BasicBuilder().device_headers():
+                with open(path, "rb") as f:
+                    h.update(f.read())
+            self._headers_digest_cache = h.digest()
+        return self._headers_digest_cache
 
     def _cached_lib(self, key: str) -> str:
         return f"{self.basic.codegen_dir}/.cache/{key}/librecom.so"
@@ -370,6 +385,10 @@ class Tuner:
         scratch = max(int(v) for v in re.findall(r"; ScratchSize: (\d+)", text))
         return vgprs, scratch
 
+    def _body_key(self, sched: ScheduleBase, params: NamedTuple) -> str:
+        """Key of a schedule body as it compiles: its emitted text and the device headers."""
+        return hashlib.sha256(sched.EmitScheduleBody(params).encode() + self._headers_digest()).hexdigest()[:24]
+
     def register_census(self, occupancy: int, tune_config: TuneConfig) -> Dict[str, Tuple[int, int]]:
         """Registers and scratch of every distinct candidate body at this occupancy, keyed by the
         body text; compiled once (``.cache/census_o{occ}.json``), ``num_processes`` at a time."""
@@ -382,7 +401,7 @@ class Tuner:
         todo: Dict[str, Tuple[ScheduleBase, NamedTuple]] = {}
         for cands in self.feat_sched_param_candidates:
             for sched, params in cands:
-                key = hashlib.sha256(sched.EmitScheduleBody(params).encode()).hexdigest()[:24]
+                key = self._body_key(sched, params)
                 if key not in census:
                     todo.setdefault(key, (sched, params))
         if todo:
@@ -406,8 +425,7 @@ class Tuner:
         limit = self.vgpr_budget(occupancy) - tune_config.census_margin
         admitted = []
         for cands in self.feat_sched_param_candidates:
-            stats = [census[hashlib.sha256(s.EmitScheduleBody(p).encode()).hexdigest()[:24]]
-                     for s, p in cands]
+            stats = [census[self._body_key(s, p)] for s, p in cands]
             keep = [k for k, (vgprs, scratch) in enumerate(stats) if scratch == 0 and vgprs <= limit]
             if not keep:
                 keep = [min(range(len(stats)), key=lambda k: (stats[k][1], stats[k][0]))]

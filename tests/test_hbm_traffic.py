@@ -29,10 +29,10 @@ def test_record_scales_by_the_copy_and_is_keyed_to_the_library(tmp_path, monkeyp
     copy_bytes = 1 << 20
     # the copy reads 1 MiB: the fetch counter shows 512 (units of 2 KiB), the write counter 1024
     fetch = _csv(tmp_path / "f_counter_collection.csv", "FETCH_SIZE",
-                 [("__amd_rocclr_copyBuffer", 512), ("__amd_rocclr_copyBuffer", 7), ("FusedKnl", 100),
+                 [("CalibrationCopyKnl", 512), ("__amd_rocclr_copyBuffer", 70000), ("FusedKnl", 100),
                   ("FusedKnl", 300), ("other", 9999)])
     write = _csv(tmp_path / "w_counter_collection.csv", "WRITE_SIZE",
-                 [("__amd_rocclr_copyBuffer", 1024), ("FusedKnl", 50), ("FusedKnl", 50)])
+                 [("CalibrationCopyKnl", 1024), ("FusedKnl", 50), ("FusedKnl", 50)])
     rec = hbm_traffic.record(model, fetch, write, copy_bytes)
     assert rec["fetch_bytes_per_unit"] == 2048 and rec["write_bytes_per_unit"] == 1024
     assert rec["read_bytes"] == 200 * 2048 and rec["written_bytes"] == 50 * 1024
@@ -48,9 +48,13 @@ def test_record_needs_both_kernels_in_the_counter_file(tmp_path, monkeypatch):
     monkeypatch.setattr(hbm_traffic, "RECORD_PATH", str(tmp_path / "hbm_traffic.json"))
     prebuilt.ensure_built("c1")
     only_fused = _csv(tmp_path / "a_counter_collection.csv", "FETCH_SIZE", [("FusedKnl", 1)])
-    both = _csv(tmp_path / "b_counter_collection.csv", "WRITE_SIZE", [("FusedKnl", 1), ("x_copyBuffer", 4)])
+    both = _csv(tmp_path / "b_counter_collection.csv", "WRITE_SIZE", [("FusedKnl", 1), ("CalibrationCopyKnl", 4)])
+    twice = _csv(tmp_path / "c_counter_collection.csv", "FETCH_SIZE",
+                 [("FusedKnl", 1), ("CalibrationCopyKnl", 4), ("CalibrationCopyKnl", 4)])
     with pytest.raises(ValueError, match="calibrate"):
         hbm_traffic.record("c1", only_fused, both, 4096)
+    with pytest.raises(ValueError, match="exactly one"):
+        hbm_traffic.record("c1", twice, both, 4096)
     with pytest.raises(ValueError, match="FETCH_SIZE"):
         hbm_traffic.record("c1", both, both, 4096)
     assert not os.path.exists(hbm_traffic.RECORD_PATH)
