@@ -57,6 +57,25 @@ def test_reference_import_lines_resolve_to_this_build():
     assert sys.modules["RecFlex.cuda_helper"] is recflex_amd.hip_helper
 
 
+SCHEDULE_IMPORT_LINES = """
+from schedules.reduce_by_key import ReduceByKeySchedule, ReduceByKeyParams
+from schedules.multi_block_per_sample import MultiBlockPerSampleSchedule, MultiBlockPerSampleParams
+from schedules.one_block_multi_sample import OneBlockMultiSampleSchedule, OneBlockMultiSampleParams
+from schedules.warp_per_sample import WarpPerSampleSchedule, WarpPerSampleParams
+from schedules.one_hot import OneHotSchedule, OneHotParams
+from schedules.one_hot_multi_block import OneHotMultiBlockSchedule, OneHotMultiBlockParams
+"""
+
+
+def test_schedule_import_lines_of_the_example_scripts_resolve():
+    """``examples/tune.py:16-21`` of the reference, run from the examples directory as there."""
+    code = ("import sys; sys.path[:0] = ['.', %r]\n" % ROOT + SCHEDULE_IMPORT_LINES +
+            "import recflex_amd.schedules as impl\n"
+            "assert OneHotSchedule is impl.OneHotSchedule and ReduceByKeyParams is impl.ReduceByKeyParams\n"
+            "assert issubclass(WarpPerSampleSchedule, impl.ScheduleBase)\n")
+    subprocess.run([sys.executable, "-c", code], cwd=f"{ROOT}/examples", check=True)
+
+
 def test_config_tuples_take_the_reference_field_names():
     from RecFlex.tuning import BasicConfig, TuneConfig
     basic = BasicConfig(batch_sizes_fname="b.txt", data_fnames=["f0.txt"], schedule_config_fname="s.txt",
