@@ -231,6 +231,9 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
     kernel_us_avg = sum(durs) / len(durs)
     kernel_us_med = durs[len(durs) // 2]
 
+    kernel_us_dense = dense_launch_us(dev, lambda: layer.forward_indices(
+        bound, tile_bytes=tile_bytes, grid_blocks=grid_blocks, xcd_segments=xcd_segments, out=outbuf))
+
     kernel_s = kernel_us_avg * 1e-6
     hbm_bytes = traffic if traffic is not None else comp_bytes
     res = {
@@ -242,6 +245,9 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
         "traffic_over_compulsory": (traffic / comp_bytes) if traffic is not None else None,
         "ms_per_step": wall / steps * 1e3,
         "kernel_us_avg": kernel_us_avg, "kernel_us_median": kernel_us_med,
+        # launch-to-launch period of a captured graph of launches: no event packets and no host
+        # between the kernels (null if the capture failed)
+        "kernel_us_dense": kernel_us_dense,
         "lookups_per_s": sum(lookups) / kernel_s,
         # whole-job rate: the K timed steps by the wall clock
         "job_algorithmic_gbps": alg_bytes / (wall / steps) / 1e9,
@@ -255,6 +261,9 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
         "grid_blocks": grid_blocks or layer.max_concurrent_blocks,
         "setup_s": round(setup_s, 2),
     }
+    ticks_model = model + "_ticks"
+    if ticks_model in prebuilt.model_names() and os.path.exists(prebuilt.lib_path(ticks_model)):
+        res["binding"] = binding_share(dev, tables, prebuilt.lib_path(ticks_model), d_idx, d_off)
     if gather_floor:
         # the memory system's floor for this batch: the same rows fetched and dropped
         from recflex_amd import gather_probe
@@ -279,6 +288,72 @@ def run_config(name: str, steps: int, warmup: int, with_cpu: bool, tile_bytes: i
     del layer, tables, d_idx, d_off, out, outbuf
     torch.cuda.empty_cache()
     return res
+
+
+TICK_NS = 10.0      # the workgroup-level entries of a timing build count the constant 100 MHz clock
+
+
+def binding_share(dev, tables, ticks_lib: str, d_idx, d_off, launches: int = 5) -> dict:
+    """The share of a workgroup's time that passes before its first tile, read from the tick
+    counters of the model's timing build (the same schedules and launch parameters with
+    clock stamps at kernel entry, after the binding and at the end of the workgroup)."""
+    import torch
+    from recflex_amd.rec_modules import FeatEmbed
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=ticks_lib)
+    bound = layer.bind_inputs(d_idx, d_off)
+    for _ in range(3):
+        layer.forward_indices(bound)
+    torch.cuda.synchronize()
+    before, total = [], []
+    for _ in range(launches):
+        layer.forward_indices(bound, timing=True)
+        b, t = layer.last_workgroup_ticks
+        before.append(b)
+        total.append(t)
+    grid = layer.max_concurrent_blocks
+    res = {"model": os.path.basename(os.path.dirname(os.path.dirname(ticks_lib))),
+           "workgroups": grid,
+           "binding_ns_per_workgroup": sum(before) / len(before) / grid * TICK_NS,
+           "total_ns_per_workgroup": sum(total) / len(total) / grid * TICK_NS,
+           "binding_share": sum(before) / sum(total)}
+    del layer
+    return res
+
+
+DENSE_LAUNCHES = 20
+
+
+def dense_launch_us(dev, launch):
+    """Microseconds per launch when DENSE_LAUNCHES launches run back to back from one captured
+    graph, two events around each replay (median of five replays).  An event pair around a
+    single launch also spans the dispatch of the kernel and the event's own packets, about two
+    microseconds that matter for a kernel of ten; this figure leaves them out."""
+    import torch
+    try:
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream(dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            launch()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(DENSE_LAUNCHES):
+                    launch()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(5):
+            s = torch.cuda.Event(enable_timing=True)
+            e = torch.cuda.Event(enable_timing=True)
+            s.record()
+            graph.replay()
+            e.record()
+            e.synchronize()
+            times.append(s.elapsed_time(e) * 1e3 / DENSE_LAUNCHES)
+        del graph
+        return sorted(times)[len(times) // 2]
+    except Exception as exc:      # the figure is an extra: never lose the run over it
+        print(f"bench.py: dense launch timing skipped ({type(exc).__name__}: {exc})", file=sys.stderr)
+        return None
 
 
 def main():
@@ -331,6 +406,8 @@ def main():
                             "output, a row counted once per lookup) / wall time per step",
         "kernel_us": head["kernel_us_avg"],
         "kernel_us_median": head["kernel_us_median"],
+        "kernel_us_dense": head["kernel_us_dense"],
+        "binding": head.get("binding"),
         "lookups_per_s": head["lookups_per_s"],
         # achieved = bytes that crossed the HBM pins per launch / FusedKnl's duration: the
         # counters' figure where it was taken on this library, else the compulsory bytes (every

@@ -74,6 +74,10 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--xcd_segments_candidates", type=str,
                         help="comma-separated tile-walk settings swept in the global stage "
                              "(-1 = flat, n > 0 = n segments per XCD)")
+    parser.add_argument("--launch_time_tolerance", type=float, default=0.0,
+                        help="global stage: launch options within this share of the fastest count "
+                             "as equally fast and the one with the fewest segments per XCD (the "
+                             "least HBM traffic) is kept; 0 = the fastest")
     parser.add_argument("--outliers", choices=["auto", "on", "off"], default="auto",
                         help="emit the optimal library with outlier tiles: bags far longer than "
                              "their feature's schedule suits are found ahead of the fused kernel "
@@ -165,6 +169,8 @@ def create_tune_config(args: argparse.Namespace) -> TuneConfig:
         kwargs["tile_bytes"] = args.tile_bytes
     if args.xcd_segments_candidates:
         kwargs["xcd_segments_candidates"] = [int(v) for v in args.xcd_segments_candidates.split(",")]
+    if args.launch_time_tolerance:
+        kwargs["launch_time_tolerance"] = args.launch_time_tolerance
     if args.tile_bytes_candidates:
         kwargs["tile_bytes_candidates"] = [int(v) for v in args.tile_bytes_candidates.split(",")]
     return TuneConfig(occupancies=occupancies, gpu_ids=gpu_ids, sm_count=sm_count,

@@ -156,8 +156,9 @@ typedef struct recom_process_args {
    * (clamped to the feature's candidate count); NULL = candidate 0 everywhere */
   const int32_t *d_schedule_choice;
   /* timing builds only: device uint64[F + 2], the kernel ADDS each feature's workgroup-ticks
-   * (s_memtime) to entries 0..F-1, the ticks every workgroup spends before its first tile (the
-   * run-time binding) to entry F and every workgroup's ticks from start to end to entry F + 1;
+   * (s_memtime, shader cycles) to entries 0..F-1 and, in units of 10 ns (the constant 100 MHz
+   * clock, s_memrealtime), the time every workgroup spends before its first tile (the run-time
+   * binding) to entry F and every workgroup's time from start to end to entry F + 1;
    * caller zeroes it.  Replaces the per-block clock() array
    * (RecFlex/code_emitter/codegen.py:301-316,388-401).  NULL runs a timing build untimed;
    * must be NULL for other builds. */

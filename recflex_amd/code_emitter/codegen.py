@@ -327,24 +327,26 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
 ''' if timing else ''
         timing_init = f'''
   __shared__ unsigned int s_ticks[NUM_FEATS];
-  const unsigned long long t_kernel_begin = d_times ? __builtin_amdgcn_s_memtime() : 0;
+  const unsigned long long t_kernel_begin = d_times ? wall_clock64() : 0;
   if (d_times)
     for (int f = threadIdx.x; f < NUM_FEATS; f += {vars_.BLOCK_THREADS}) s_ticks[f] = 0;
 ''' if timing else ''
         # ticks every workgroup spends before its first tile (the binding), entry NUM_FEATS
         timing_bound = '''
-  const unsigned long long t_bound = d_times ? __builtin_amdgcn_s_memtime() : 0;
+  const unsigned long long t_bound = d_times ? wall_clock64() : 0;
 ''' if timing else ''
         timing_flush = f'''
   if (d_times) {{
     __syncthreads();
+    // the workgroup's end: before the counters are flushed, which is not part of its work
+    const unsigned long long t_kernel_end = wall_clock64();
     for (int f = threadIdx.x; f < NUM_FEATS; f += {vars_.BLOCK_THREADS})
       if (s_ticks[f]) atomicAdd(&d_times[f], static_cast<unsigned long long>(s_ticks[f]));
     if (threadIdx.x == 0) {{
-      // beyond the per-feature entries: the workgroup's ticks before its first tile, and all of
-      // its ticks
+      // beyond the per-feature entries, on the constant 100 MHz clock (10 ns; the per-feature
+      // ticks count shader cycles): the workgroup's time before its first tile, and all of it
       atomicAdd(&d_times[NUM_FEATS], t_bound - t_kernel_begin);
-      atomicAdd(&d_times[NUM_FEATS + 1], __builtin_amdgcn_s_memtime() - t_kernel_begin);
+      atomicAdd(&d_times[NUM_FEATS + 1], t_kernel_end - t_kernel_begin);
     }}
   }}
 ''' if timing else ''

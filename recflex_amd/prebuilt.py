@@ -8,6 +8,9 @@ its library is missing.  Names:
 ``cN_tuned``       CN with the schedules, occupancy and launch parameters recorded in
                    ``recflex_amd/tuned/cN_schedule.json`` (written by ``examples/tune.py``); the
                    default build if that file is absent
+``cN_tuned_ticks`` c2_tuned / c3_tuned as timing builds (tick counters at kernel entry, after the
+                   binding and at the end of each workgroup): ``bench.py`` reads the binding's
+                   share of a workgroup's time from them
 ``c1_o2``, ``c1_o5`` C1 built for 2 and 5 workgroups per CU (its light kernel reaches 8 by
                    itself, so the dynamic-LDS pad has to hold the others off)
 ``c3_flat``        C3 with the flat tile walk instead of the XCD-segmented one (for comparison)
@@ -104,6 +107,10 @@ def _tuned(wl: Workload, fname: str) -> ModelSpec:
     if isinstance(doc, dict) and doc.get("outliers"):
         kwargs["outliers"] = True
     return ModelSpec(wl, fs, occupancy, kwargs)
+
+
+def _with_ticks(spec: ModelSpec) -> ModelSpec:
+    return spec._replace(emit_kwargs=dict(spec.emit_kwargs, timing=True))
 
 
 def _variants() -> ModelSpec:
@@ -243,6 +250,10 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c3_tuned": lambda: _tuned(make_workload("C3"), "c3_schedule.json"),
     "c4_tuned": lambda: _tuned(make_workload("C4"), "c4_schedule.json"),
     "c5_tuned": lambda: _tuned(make_workload("C5"), "c5_schedule.json"),
+    # c2_tuned / c3_tuned with the tick counters of a timing build: the share of a workgroup's
+    # time that passes before its first tile (the binding), reported by bench.py
+    "c2_tuned_ticks": lambda: _with_ticks(_tuned(make_workload("C2"), "c2_schedule.json")),
+    "c3_tuned_ticks": lambda: _with_ticks(_tuned(make_workload("C3"), "c3_schedule.json")),
     "c1_o2": lambda: _default(make_workload("C1"), occupancy=2),
     "c1_o5": lambda: _default(make_workload("C1"), occupancy=5),
     "c3_flat": lambda: _default(make_workload("C3"), xcd_aware=False),

@@ -138,8 +138,8 @@ class FeatEmbed(nn.Module):
             torch.cuda.synchronize(self.device)
 
         self.output_units = self.lib.embed_dim_sum
-        # timing builds: (ticks before the first tile, ticks in all) summed over the workgroups
-        # of the last timed launch
+        # timing builds: (time before the first tile, time in all) summed over the workgroups of
+        # the last timed launch, in units of 10 ns (the constant 100 MHz clock)
         self.last_workgroup_ticks = None
         self._io_cache_key = None
         self._io_bound = None
@@ -186,8 +186,8 @@ class FeatEmbed(nn.Module):
         if timing:
             if not self.lib.info.timing:
                 raise RuntimeError("timing=True needs a library emitted with timing=True")
-            # per-feature ticks, then the workgroups' ticks before their first tile, then all
-            # of their ticks (kept in self.last_workgroup_ticks)
+            # per-feature ticks (shader cycles), then the workgroups' time before their first
+            # tile and all of their time in units of 10 ns (kept in self.last_workgroup_ticks)
             times = torch.zeros([self.lib.num_features + 2], dtype=torch.int64, device=self.device)
         if schedule_choice is not None:
             if schedule_choice.dtype != torch.int32 or schedule_choice.numel() != len(self.embed_tables) \

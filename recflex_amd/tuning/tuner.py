@@ -105,6 +105,13 @@ class TuneConfig(NamedTuple):
     # global stage: L2-locality settings of the tile walk to try (launch parameter
     # xcd_segments; -1 = flat walk); empty = only the emitted default
     xcd_segments_candidates: List[int] = []
+    # global stage: launch options whose time is within this share of a contender's fastest count
+    # as equally fast, and of those the one with the fewest segments per XCD wins (fewer segments
+    # = fewer L2s that fetch a feature's hot rows = less HBM traffic: C3 fetches 478 MB at 10
+    # segments, 494 MB at 12, 512 MB at 16 and 541 MB at 24, in 119.7 / 119.9 / 118.2 / 118.2 us).
+    # 0 = the fastest option wins; a deployment that shares the memory system with other kernels
+    # may give away a per cent of time for the traffic
+    launch_time_tolerance: float = 0.0
     # global stage: also time the untuned default schedules at every occupancy and keep them
     # if they win (tile times measured feature by feature do not always add up to kernel time)
     include_default: bool = True
@@ -112,6 +119,20 @@ class TuneConfig(NamedTuple):
 
 def padded_sched_num(orig_num: int, max_concurrent_blocks: int) -> int:
     return (orig_num + max_concurrent_blocks - 1) // orig_num * orig_num
+
+
+def pick_launch_option(launch_opts: List[Tuple[int, int]], times: List[float],
+                       tolerance: float) -> int:
+    """Index of the launch option (tile_bytes, xcd_segments) to keep: the fastest, unless options
+    with fewer (positive) segments per XCD are within ``tolerance`` of it -- then the one with the
+    fewest segments among those, the faster one on a tie.  The flat walk (segments <= 0) fetches
+    the most and never wins a tie."""
+    best = int(np.argmin(times))
+    if launch_opts[best][1] <= 0:
+        return best
+    limit = times[best] * (1.0 + tolerance)
+    near = [k for k, (_, xs) in enumerate(launch_opts) if xs > 0 and times[k] <= limit]
+    return min(near, key=lambda k: (launch_opts[k][1], times[k]))
 
 
 class Tuner:
@@ -725,11 +746,14 @@ class Tuner:
         times, best_opts = [], []
         for output_dir, occupancy, _ in contenders:
             per_opt = [self._read_kernel_time(output_dir, tune_config, tb, xs) for tb, xs in launch_opts]
-            k = int(np.argmin(per_opt))
-            times.append(per_opt[k])
+            # contenders compete on their fastest option; the tolerance rule then settles the
+            # launch option of the winner only (kept and fastest option differ by at most the
+            # tolerance, which must not decide between contenders)
+            times.append(float(np.min(per_opt)))
+            k = pick_launch_option(launch_opts, per_opt, tune_config.launch_time_tolerance)
             best_opts.append(launch_opts[k])
             kind = "default" if "/default/o" in output_dir else "tuned"
-            print(f"occupancy: {occupancy} ({kind}), t(ns): {per_opt[k]}"
+            print(f"occupancy: {occupancy} ({kind}), t(ns): {times[-1]}"
                   + (f", (tile_bytes, xcd_segments): {launch_opts[k]} (of "
                      f"{ {o: round(t) for o, t in zip(launch_opts, per_opt)} })" if len(launch_opts) > 1 else ""))
 

@@ -366,3 +366,18 @@ def test_kernel_trace_parser_groups_calls_and_takes_medians(tmp_path):
         parse_knl_batch_times("FusedKnl", str(path), passes=4)
     with pytest.raises(FileNotFoundError):
         parse_knl_call_durations("FusedKnl", str(tmp_path / "nothing"))
+
+
+def test_launch_option_ties_go_to_the_fewest_segments():
+    from recflex_amd.tuning.tuner import pick_launch_option
+    opts = [(65536, -1), (65536, 1), (65536, 8), (65536, 10), (65536, 12), (65536, 16), (65536, 24)]
+    times = [120.0, 131.7, 125.6, 119.7, 119.9, 118.2, 118.2]
+    assert opts[pick_launch_option(opts, times, 0.015)] == (65536, 10)     # within 1.5 % of 118.2
+    assert opts[pick_launch_option(opts, times, 0.0)] == (65536, 16)       # no tolerance: the fastest
+    assert opts[pick_launch_option(opts, times, 0.2)] == (65536, 1)
+    # the flat walk wins only by being the fastest, and is never preferred on a tie
+    assert opts[pick_launch_option(opts, [100.0] + times[1:], 0.015)] == (65536, -1)
+    assert opts[pick_launch_option(opts, [118.3] + times[1:], 0.015)] == (65536, 10)
+    # two tile sizes at the same segment count: the faster of the two
+    opts2 = [(32768, 8), (65536, 8), (65536, 16)]
+    assert opts2[pick_launch_option(opts2, [101.0, 100.5, 100.0], 0.015)] == (65536, 8)
