@@ -24,6 +24,8 @@ Three byte counts per launch, because Zipf-hot rows are served from the caches:
 
 ``roofline.frac`` = HBM bytes per launch / kernel time / 8 TB/s, with the measured traffic where
 it is known and the compulsory bytes (a lower bound of the traffic) otherwise; it cannot exceed 1.
+``roofline.random_line_gbps`` is the rate at which the same device fetches 128-byte lines at
+uniformly random addresses (measured in the same run): the ceiling for a gather without reuse.
 """
 
 import argparse
@@ -320,6 +322,28 @@ def binding_share(dev, tables, ticks_lib: str, d_idx, d_off, launches: int = 5) 
     return res
 
 
+RANDOM_LINE_ROWS = 1 << 24          # x 128 bytes = 2 GiB
+
+
+def random_line_gbps(dev, steps: int) -> float:
+    """GB/s at which this device fetches 128-byte lines at uniformly random addresses of a 2 GiB
+    table (every lookup one whole line, 16 Mi lookups, the gather probe at its fastest setting):
+    the ceiling of the memory system for a gather without any reuse, measured live, to be read
+    beside the 8 TB/s that sequential traffic reaches at the pins."""
+    import torch
+    from recflex_amd.gather_probe import GatherProbe
+    table = torch.zeros((RANDOM_LINE_ROWS, 32), dtype=torch.float32, device=dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4711)
+    idx = torch.randint(0, RANDOM_LINE_ROWS, (RANDOM_LINE_ROWS,), dtype=torch.int32, device=dev,
+                        generator=gen)
+    probe = GatherProbe(dev, [table], [idx], [128])
+    best = probe.best_time_us(steps=min(steps, 10))
+    del probe, table, idx
+    torch.cuda.empty_cache()
+    return RANDOM_LINE_ROWS * 128 / (best["us"] * 1e-6) / 1e9
+
+
 DENSE_LAUNCHES = 20
 
 
@@ -420,6 +444,10 @@ def main():
                      "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
                      "algorithmic_gbps": head["algorithmic_gbps"]},
     }
+    if floor:
+        # what a gather without reuse reaches on this device, and the kernel's HBM rate against it
+        line["roofline"]["random_line_gbps"] = random_line_gbps(torch.device("cuda", 0), args.steps)
+        line["roofline"]["frac_of_random_line_rate"] = head["hbm_gbps"] / line["roofline"]["random_line_gbps"]
     if "gather_floor_us" in head:
         # time of the bare fetch of the same rows (gather probe): what the memory system allows
         line["roofline"]["gather_floor_us"] = head["gather_floor_us"]

@@ -35,13 +35,15 @@ RECORD_PATH = os.path.join(prebuilt.TUNED_DIR, "hbm_traffic.json")
 
 
 def library_key(model: str) -> Optional[str]:
-    """Key of what the model's library is built from: its emitted ``process.hip`` and the device
-    headers.  ``None`` if the model was never emitted here."""
+    """Key of what the model's kernels are built from: its emitted ``process.hip`` and the
+    device-code headers (``csrc/include/*.h``; the C-ABI header only shapes host code).  ``None``
+    if the model was never emitted here."""
     src = os.path.join(prebuilt.model_dir(model), "process.hip")
     if not os.path.exists(src):
         return None
+    basic = BasicBuilder()
     h = hashlib.sha256()
-    for path in [src] + BasicBuilder().device_headers():
+    for path in [src] + [p for p in basic.device_headers() if os.path.dirname(p) == basic.include]:
         with open(path, "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:24]
