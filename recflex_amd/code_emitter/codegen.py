@@ -27,6 +27,17 @@ from .build_basic import BasicBuilder
 
 # memory traffic (bytes) the run-time binding aims at per tile
 DEFAULT_TILE_BYTES = 64 * 1024
+SIMDS_PER_CU = 4
+MAX_WAVES_PER_SIMD = 8
+
+
+def waves_per_simd(occupancy: int, block_threads: int) -> int:
+    """Wavefronts each SIMD of a CU holds when ``occupancy`` workgroups of ``block_threads``
+    threads are resident on it."""
+    waves = occupancy * ((block_threads + 63) // 64)
+    return max(1, min(MAX_WAVES_PER_SIMD, -(-waves // SIMDS_PER_CU)))
+
+
 # XCDs (L2 slices) of an MI355X; workgroup i of a launch runs on XCD i % 8
 XCD_COUNT = 8
 # per-bag traffic that does not depend on the bag length, besides the output slice: one offset
@@ -362,7 +373,11 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
             f"      case {feat_idx}: ProcessFeat{feat_idx}({call_args}); break;\n"
             for feat_idx in body_ids)
 
-        launch_bounds = (f"__launch_bounds__({vars_.BLOCK_THREADS}, {occupancy})" if occupancy
+        # the register budget that lets `occupancy` workgroups share a CU: hipcc reads the second
+        # argument of __launch_bounds__ as wavefronts per SIMD, not workgroups per CU (the two are
+        # the same number only for 256-thread workgroups on four SIMDs)
+        launch_bounds = (f"__launch_bounds__({vars_.BLOCK_THREADS}, "
+                         f"{waves_per_simd(occupancy, self.block_threads)})" if occupancy
                          else f"__launch_bounds__({vars_.BLOCK_THREADS})")
         if bind_once:
             bind_decl = "  __shared__ rfx::PrefixStorage<NUM_FEATS> s_bind;\n"

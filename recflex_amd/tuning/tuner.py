@@ -31,7 +31,8 @@ from typing import Dict, List, NamedTuple, Optional, Sequence, Tuple
 import numpy as np
 
 from recflex_amd.code_emitter import CodeEmitter, ScheduleBase, MetaData
-from recflex_amd.code_emitter.codegen import BAG_FIXED_BYTES, DEFAULT_TILE_BYTES, INDEX_BYTES
+from recflex_amd.code_emitter.codegen import (BAG_FIXED_BYTES, DEFAULT_TILE_BYTES, INDEX_BYTES,
+                                               waves_per_simd)
 from recflex_amd.utils import compile_build, os_check
 from recflex_amd.task_manager import TaskManager
 from recflex_amd.parser import (parse_raw_data_batches, parse_table_shapes, parse_table_dtypes,
@@ -378,10 +379,11 @@ class Tuner:
     # ---- register census ----------------------------------------------------------------------
 
     @staticmethod
-    def vgpr_budget(occupancy: int) -> int:
-        """Vector registers per lane that ``occupancy`` 256-thread workgroups per CU (one
-        wavefront per SIMD each) leave a kernel on gfx950: 512 per SIMD in blocks of 8."""
-        return min(512, 512 // max(1, occupancy) // 8 * 8)
+    def vgpr_budget(occupancy: int, block_threads: int = 256) -> int:
+        """Vector registers per lane that ``occupancy`` workgroups of ``block_threads`` threads per
+        CU leave a kernel on gfx950: 512 per SIMD in blocks of 8, shared by the wavefronts the
+        SIMD then holds (one per 256-thread workgroup)."""
+        return min(512, 512 // waves_per_simd(max(1, occupancy), block_threads) // 8 * 8)
 
     def _census_one(self, sched_param: Tuple[ScheduleBase, NamedTuple], occupancy: int,
                     tune_config: TuneConfig) -> Tuple[int, int]:
@@ -443,7 +445,7 @@ class Tuner:
         if not tune_config.register_census:
             return [list(range(len(c))) for c in self.feat_sched_param_candidates]
         census = self.register_census(occupancy, tune_config)
-        limit = self.vgpr_budget(occupancy) - tune_config.census_margin
+        limit = self.vgpr_budget(occupancy, self.basic.block_threads) - tune_config.census_margin
         admitted = []
         for cands in self.feat_sched_param_candidates:
             stats = [census[self._body_key(s, p)] for s, p in cands]

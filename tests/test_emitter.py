@@ -240,3 +240,18 @@ def test_outlier_tiles_are_emitted_on_request():
     assert "#define RFX_OUTLIERS 0" in plain and "OutlierKnl" not in plain and "c_long_thr" not in plain
     with pytest.raises(AssertionError):
         em.emit_kernel(occupancy=4, outliers=True, timing=True)
+
+
+def test_launch_bounds_carry_wavefronts_per_simd_not_workgroups_per_cu():
+    """hipcc reads the second argument of __launch_bounds__ as wavefronts per SIMD: a build of
+    64-thread workgroups at 20 per CU has to ask for 5, one of 128-thread workgroups at 6 for 3."""
+    from recflex_amd.code_emitter.codegen import waves_per_simd
+    from recflex_amd.tuning.tuner import Tuner
+    assert [waves_per_simd(o, 256) for o in (1, 2, 4, 5, 8, 12)] == [1, 2, 4, 5, 8, 8]
+    assert waves_per_simd(20, 64) == 5 and waves_per_simd(16, 64) == 4 and waves_per_simd(6, 128) == 3
+    assert waves_per_simd(1, 64) == 1 and waves_per_simd(2, 512) == 4
+    assert Tuner.vgpr_budget(5) == 96 and Tuner.vgpr_budget(4) == 128 and Tuner.vgpr_budget(6) == 80
+    assert Tuner.vgpr_budget(20, 64) == 96 and Tuner.vgpr_budget(6, 128) == 168
+    fs = [default_schedule(MetaData(32, "float"), 4, 64)]
+    src = CodeEmitter(fs).emit_kernel(occupancy=20)
+    assert "constexpr int BLOCK_THREADS = 64;" in src and "__launch_bounds__(BLOCK_THREADS, 5)" in src
