@@ -63,8 +63,9 @@ typedef struct recom_info {
   int32_t reserved[3];
 } recom_info;
 
-#define RECOM_ABI_VERSION 4     /* 4: recom_process_static_workspace; the once-per-launch binding
-                                 * table of very wide models moved into the workspace */
+#define RECOM_ABI_VERSION 5     /* 4: recom_process_static_workspace; the once-per-launch binding
+                                 * table of very wide models moved into the workspace
+                                 * 5: recom_process_args.start_event / stop_event */
 
 /* largest workspace recom_process_static_workspace serves from the library's static array */
 #define RECOM_STATIC_WORKSPACE_MAX_BYTES (32 * 1024 * 1024)
@@ -182,6 +183,15 @@ typedef struct recom_process_args {
    * (RecFlex/code_emitter/codegen.py:403-444, RecFlex/rec_modules.py:44-52). */
   void *d_workspace;
   int64_t workspace_bytes;
+  /* hipEvent_t (created by the caller with timing enabled) or NULL.  When either is given, the
+   * fused kernel is launched with hipExtLaunchKernel and the events receive the begin and the end
+   * of that very dispatch -- the kernel's own duration, without the dispatch latency and the
+   * marker packets that a pair of hipEventRecord calls around the launch adds (about two
+   * microseconds, which matter for a kernel of ten).  Kernels launched ahead of the fused one
+   * (outlier search, once-per-launch binding) are outside the pair.  Not for use under stream
+   * capture.  The reference times with the profiler only (RecFlex/cuda_helper.py:33-51). */
+  void *start_event;
+  void *stop_event;
 } recom_process_args;
 
 /* Launch the fused kernel: for every feature f and sample b,

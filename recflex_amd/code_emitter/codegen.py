@@ -580,8 +580,15 @@ static int launch_kernels(const recom_process_args *a, void *workspace) {
       const_cast<int32_t **>(&a->d_schedule_choice),
       const_cast<unsigned long long **>(&a->d_times), &stride_arg, &bound, &workspace,
       &outlier_space};
-  e = hipLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
-                      kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream));
+  if (a->start_event || a->stop_event)
+    // the events take the begin and end timestamps of this very dispatch
+    e = hipExtLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
+                           kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream),
+                           static_cast<hipEvent_t>(a->start_event),
+                           static_cast<hipEvent_t>(a->stop_event), 0);
+  else
+    e = hipLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
+                        kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream));
   return static_cast<int>(e);
 }
 

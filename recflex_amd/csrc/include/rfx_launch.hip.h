@@ -8,6 +8,7 @@
 // a little more than 1/(occupancy + 1) of it per workgroup.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <mutex>
 #include <stdint.h>
 

@@ -105,6 +105,49 @@ class HipProfiler:
         self._call("hipProfilerStop")
 
 
+class HipEvent:
+    """A ``hipEvent_t`` with timing enabled, for the ``start_event`` / ``stop_event`` of
+    ``recom_process``: the library hands the pair to ``hipExtLaunchKernel``, which stamps them
+    with the begin and end of the fused kernel's own dispatch.  ``handle`` is the raw event."""
+
+    _hip = None
+
+    def __init__(self):
+        if HipEvent._hip is None:
+            hip = _load_hip()
+            hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+            hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+            hip.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+            hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p,
+                                                ctypes.c_void_p]
+            hip.hipGetErrorString.restype = ctypes.c_char_p
+            HipEvent._hip = hip
+        ev = ctypes.c_void_p()
+        self._check(self._hip.hipEventCreate(ctypes.byref(ev)), "hipEventCreate")
+        self.handle = ev.value
+
+    @classmethod
+    def _check(cls, ret: int, what: str) -> None:
+        if ret != HIP_SUCCESS:
+            msg = cls._hip.hipGetErrorString(ret)
+            raise RuntimeError(f"{what}: hipError_t {ret} ({msg.decode() if msg else '?'})")
+
+    def synchronize(self) -> None:
+        self._check(self._hip.hipEventSynchronize(self.handle), "hipEventSynchronize")
+
+    def elapsed_us(self, later: "HipEvent") -> float:
+        """Microseconds from this event to ``later`` (both must have completed)."""
+        ms = ctypes.c_float()
+        self._check(self._hip.hipEventElapsedTime(ctypes.byref(ms), self.handle, later.handle),
+                    "hipEventElapsedTime")
+        return ms.value * 1e3
+
+    def __del__(self):
+        if getattr(self, "handle", None) and self._hip is not None:
+            self._hip.hipEventDestroy(self.handle)
+            self.handle = None
+
+
 # names of the reference module, for scripts written against it
 CudaInfoQuerier = HipInfoQuerier
 CudaProfiler = HipProfiler

@@ -165,7 +165,7 @@ class FeatEmbed(nn.Module):
 
     def _launch(self, batch: int, timing: bool, timing_schedules: Optional[int], tile_bytes: int,
                 grid_blocks: int, schedule_choice: torch.Tensor = None, out: torch.Tensor = None,
-                xcd_segments: int = 0, **inputs):
+                xcd_segments: int = 0, kernel_events=None, **inputs):
         row_stride = 0
         if out is not None:
             if out.dtype != torch.float32 or out.numel() != batch * self.output_units \
@@ -195,6 +195,8 @@ class FeatEmbed(nn.Module):
                 raise TypeError("schedule_choice must be an int32 device tensor with one entry per feature")
             inputs["schedule_choice"] = schedule_choice.data_ptr()
         stream = torch.cuda.current_stream(self.device).cuda_stream
+        if kernel_events is not None:
+            inputs.update(start_event=kernel_events[0].handle, stop_event=kernel_events[1].handle)
         if self.workspace is not None:
             inputs.update(workspace=self.workspace.data_ptr(),
                           workspace_bytes=self.workspace.numel() * 4)
@@ -280,12 +282,13 @@ class FeatEmbed(nn.Module):
                         offsets: Sequence[torch.Tensor] = None,
                         timing: bool = False, timing_schedules: int = None, tile_bytes: int = 0,
                         grid_blocks: int = 0, schedule_choice: torch.Tensor = None,
-                        out: torch.Tensor = None, xcd_segments: int = 0):
+                        out: torch.Tensor = None, xcd_segments: int = 0, kernel_events=None):
         """Per-feature int32 device tensors ``indices[f]`` (``[L_f]``) and ``offsets[f]``
         (``[batch + 1]``, exclusive prefix sums, ``offsets[f][0] == 0``) -> ``[batch, sum(dim)]``
         fp32 (with ``timing=True``: ``(output, task_times)``).  ``out``: write into this
         preallocated tensor instead of allocating one.  Instead of the two lists, the result of
-        ``bind_inputs`` may be given."""
+        ``bind_inputs`` may be given.  ``kernel_events``: a pair of ``hip_helper.HipEvent`` that
+        receives the begin and end of the fused kernel's own dispatch."""
         if isinstance(indices, BoundInputs):
             bound = indices
         else:
@@ -302,7 +305,7 @@ class FeatEmbed(nn.Module):
         batch = bound.batch
         res = self._launch(batch, timing, timing_schedules, tile_bytes, grid_blocks,
                            schedule_choice=schedule_choice, out=out, xcd_segments=xcd_segments,
-                           io_ptrs=bound.io_ptrs.data_ptr())
+                           kernel_events=kernel_events, io_ptrs=bound.io_ptrs.data_ptr())
         if timing:
             return res[0].view(batch, self.output_units), res[1]
         return res.view(batch, self.output_units)

@@ -490,3 +490,40 @@ def test_two_libraries_write_column_slabs_of_one_buffer():
     d_off = [torch.from_numpy(o).to(dev) for o in offsets]
     with pytest.raises(RecomError):
         layer.forward_indices(d_idx, d_off, out=whole[:, 2:2 + widths[0]])
+
+
+@pytest.mark.parametrize("name", ["c3s", "wider", "c3s_outliers"])
+def test_kernel_events_take_the_dispatch_time_and_change_nothing(name):
+    """``start_event`` / ``stop_event`` of the C ABI: the launch goes through
+    ``hipExtLaunchKernel``, the output keeps its bits, and the pair reads a duration that is
+    positive and no longer than a pair of event records around the same launch."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.hip_helper import HipEvent
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    wl = prebuilt.model_spec(name).workload
+    dev = torch.device("cuda", 0)
+    print(f"[case] kernel events model={name} F={wl.num_features} B={wl.batch}", flush=True)
+    tables = gen_tables(wl, dev)
+    indices, offsets = gen_inputs(wl)
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib(name))
+    bound = layer.bind_inputs([torch.from_numpy(i).to(dev) for i in indices],
+                              [torch.from_numpy(o).to(dev) for o in offsets])
+    plain = layer.forward_indices(bound).clone()
+    torch.cuda.synchronize()
+    inside, around = [], []
+    for _ in range(5):
+        pair = (HipEvent(), HipEvent())
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        timed = layer.forward_indices(bound, kernel_events=pair)
+        e.record()
+        torch.cuda.synchronize()
+        assert torch.equal(timed.view(torch.int32), plain.view(torch.int32))
+        inside.append(pair[0].elapsed_us(pair[1]))
+        around.append(s.elapsed_time(e) * 1e3)
+    print(f"   dispatch {min(inside):.2f} us, event records around it {min(around):.2f} us", flush=True)
+    assert all(0.0 < t < 1e5 for t in inside)
+    assert min(inside) <= min(around) * 1.05
