@@ -91,6 +91,9 @@ constexpr int kBindMaxSplitTiles = 2048;
 // a tile is rounded up to one whole workgroup pass of its schedule only if that pass carries at
 // most this many times the target traffic per tile
 constexpr int kMaxTileFactor = 8;
+// ... or, whatever it carries, if whole passes still give the grid this many tiles per workgroup
+// (estimated from the feature at hand: its whole passes times the number of features)
+constexpr int kPlentyTilesPerWorkgroup = 2;
 
 // Models of up to this many features also keep, per feature, the three addresses a tile needs
 // (table, indices, offsets) in LDS: the binding reads them anyway, and a tile then starts with
@@ -316,10 +319,18 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     } else if (B > 0) {
       bpt = (B + tiles - 1) / tiles;
       // Tiles are whole workgroup passes (g bags) -- unless one pass of this schedule is more
-      // than kMaxTileFactor times the traffic a tile should carry: then the tile keeps its
-      // share of the traffic and some of the schedule's teams idle.
+      // than kMaxTileFactor times the traffic a tile should carry AND whole passes would leave
+      // the grid short of tiles: then the tile keeps its share of the traffic and some of the
+      // schedule's teams idle (a small batch is spread over more workgroups that way).  With
+      // tiles in plenty -- this feature's whole passes times the number of features is at
+      // least kPlentyTilesPerWorkgroup tiles per workgroup of the grid -- idle teams are a pure
+      // loss: a batch whose bags are twice as long as the tile size was chosen for ran 262 us
+      // with a quarter of the wavefronts busy in the long-bag features, 197 us with whole passes.
       const int whole = (bpt + g - 1) / g * g;
-      if (fixed_tiles || bpt >= g ||
+      const bool plenty = grid_blocks > 0 &&
+                          static_cast<int64_t>(B / g) * F >=
+                              static_cast<int64_t>(kPlentyTilesPerWorkgroup) * grid_blocks;
+      if (fixed_tiles || bpt >= g || plenty ||
           static_cast<int64_t>(whole) * bag_cost <= static_cast<int64_t>(kMaxTileFactor) * tile_size)
         bpt = whole;
       tiles = (B + bpt - 1) / bpt;

@@ -11,6 +11,9 @@ its library is missing.  Names:
 ``cN_tuned_ticks`` c2_tuned / c3_tuned as timing builds (tick counters at kernel entry, after the
                    binding and at the end of each workgroup): ``bench.py`` reads the binding's
                    share of a workgroup's time from them
+``c3_tuned_static`` c3_tuned with the tiles per feature frozen at emit time to what the run-time
+                   binding chooses for the benchmark batch (the reference's fixed-thread-binding
+                   ablation, ``examples/ablation_fixed_binding.py``)
 ``c1_o2``, ``c1_o5`` C1 built for 2 and 5 workgroups per CU (its light kernel reaches 8 by
                    itself, so the dynamic-LDS pad has to hold the others off)
 ``c3_flat``        C3 with the flat tile walk instead of the XCD-segmented one (for comparison)
@@ -107,6 +110,23 @@ def _tuned(wl: Workload, fname: str) -> ModelSpec:
     if isinstance(doc, dict) and doc.get("outliers"):
         kwargs["outliers"] = True
     return ModelSpec(wl, fs, occupancy, kwargs)
+
+
+def _frozen_binding(spec: ModelSpec) -> ModelSpec:
+    """The model with the tiles per feature frozen at emit time to what the run-time binding
+    chooses for the workload's own (seeded) batch: the fixed-thread-binding ablation."""
+    from .code_emitter.codegen import BAG_FIXED_BYTES, DEFAULT_TILE_BYTES, INDEX_BYTES
+    from .tuning.measure import tiles_per_feature
+    from .workloads import gen_inputs
+    _, offsets = gen_inputs(spec.workload)
+    metas = [s.meta for s, _ in spec.feat_schedules]
+    counts = tiles_per_feature(offsets, [m.row_bytes + INDEX_BYTES for m in metas],
+                               [m.embed_dim * 4 + BAG_FIXED_BYTES for m in metas],
+                               [s.TileGranularity(p) for s, p in spec.feat_schedules],
+                               spec.emit_kwargs.get("tile_bytes") or DEFAULT_TILE_BYTES,
+                               grid_blocks=TUNE_FIXTURE_SM_COUNT * (spec.occupancy or DEFAULT_OCCUPANCY))
+    return spec._replace(emit_kwargs=dict(spec.emit_kwargs,
+                                          fixed_task_block_nums=[max(1, c) for c in counts]))
 
 
 def _with_ticks(spec: ModelSpec) -> ModelSpec:
@@ -254,6 +274,8 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     # time that passes before its first tile (the binding), reported by bench.py
     "c2_tuned_ticks": lambda: _with_ticks(_tuned(make_workload("C2"), "c2_schedule.json")),
     "c3_tuned_ticks": lambda: _with_ticks(_tuned(make_workload("C3"), "c3_schedule.json")),
+    # c3_tuned with its binding frozen for the benchmark batch (examples/ablation_fixed_binding.py)
+    "c3_tuned_static": lambda: _frozen_binding(_tuned(make_workload("C3"), "c3_schedule.json")),
     "c1_o2": lambda: _default(make_workload("C1"), occupancy=2),
     "c1_o5": lambda: _default(make_workload("C1"), occupancy=5),
     "c3_flat": lambda: _default(make_workload("C3"), xcd_aware=False),

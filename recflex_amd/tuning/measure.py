@@ -432,6 +432,7 @@ class KernelTimer:
 
 
 MAX_TILE_FACTOR = 8      # rfx::kMaxTileFactor
+PLENTY_TILES_PER_WORKGROUP = 2                      # rfx::kPlentyTilesPerWorkgroup
 AUTO_TILES_PER_WORKGROUP = 64                       # rfx::kAutoTilesPerWorkgroup
 AUTO_TILE_MIN, AUTO_TILE_MAX = 64 * 1024, 256 * 1024    # rfx::kAutoTileMin / kAutoTileMax
 AUTO_TILE_FLOOR = 4 * 1024                              # rfx::kAutoTileFloor
@@ -457,11 +458,15 @@ def auto_tile_bytes(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int],
 
 
 def tiles_per_feature(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int],
-                      bag_bytes: Sequence[int], gran: Sequence[int], tile_bytes: int) -> List[int]:
+                      bag_bytes: Sequence[int], gran: Sequence[int], tile_bytes: int,
+                      grid_blocks: int = 0) -> List[int]:
     """Host restatement of the device binding (``rfx::bind_tiles``): tiles each feature gets
-    for this batch.  A schedule that can split bags over workgroups (granularity -1) counts as
-    one bag per workgroup pass: a binding frozen at emit time never splits."""
+    for this batch on a grid of ``grid_blocks`` workgroups (0: unknown, taken as too large for
+    the whole-pass rule of plentiful tiles to apply).  A schedule that can split bags over
+    workgroups (granularity -1) counts as one bag per workgroup pass: a binding frozen at emit
+    time never splits."""
     out = []
+    num_feats = len(offsets)
     for off, lb, bb, g in zip(offsets, lookup_bytes, bag_bytes, gran):
         g = 1 if g < 0 else g
         batch = len(off) - 1
@@ -472,7 +477,8 @@ def tiles_per_feature(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int]
         tiles = min(max(-(-cost // tile_bytes), 1), batch)
         bpt = -(-batch // tiles)
         whole = -(-bpt // g) * g
-        if bpt >= g or whole * (cost // batch) <= MAX_TILE_FACTOR * tile_bytes:
+        plenty = grid_blocks > 0 and (batch // g) * num_feats >= PLENTY_TILES_PER_WORKGROUP * grid_blocks
+        if bpt >= g or plenty or whole * (cost // batch) <= MAX_TILE_FACTOR * tile_bytes:
             bpt = whole
         out.append(-(-batch // bpt))
     return out

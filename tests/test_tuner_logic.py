@@ -381,3 +381,15 @@ def test_launch_option_ties_go_to_the_fewest_segments():
     # two tile sizes at the same segment count: the faster of the two
     opts2 = [(32768, 8), (65536, 8), (65536, 16)]
     assert opts2[pick_launch_option(opts2, [101.0, 100.5, 100.0], 0.015)] == (65536, 8)
+
+
+def test_whole_passes_when_tiles_are_plentiful():
+    """A pass of 4 bags of 160 KB each is more than 8 tiles of 64 KiB: on a small batch the tile
+    stays below a pass (more workgroups get work), on a batch whose whole passes already give
+    every workgroup of the grid two tiles it is a whole pass (no idle teams)."""
+    off = np.arange(0, 2049 * 320, 320, dtype=np.int64)          # 2 048 bags of 320 lookups
+    args = ([off] * 100, [516] * 100, [516] * 100, [4] * 100, 65536)
+    assert tiles_per_feature(*args)[0] == 2048                   # grid unknown: one bag per tile
+    assert tiles_per_feature(*args, grid_blocks=1280)[0] == 512  # 512 * 100 >= 2 * 1280
+    few = ([off[:33]] * 4, [516] * 4, [516] * 4, [4] * 4, 65536)
+    assert tiles_per_feature(*few, grid_blocks=1280)[0] == 32    # 8 * 4 < 2 * 1280: spread out
