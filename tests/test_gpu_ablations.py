@@ -219,3 +219,31 @@ def test_end_to_end_measure_returns_a_positive_time():
     print("[case] end_to_end.measure over", len(raw_batches), "batches", flush=True)
     t_ms = e2e.measure(preprocess, model, model.embed_layer.max_concurrent_blocks, raw_batches)
     assert np.isfinite(t_ms) and t_ms > 0
+
+
+def test_frozen_binding_example_gives_the_bits_of_the_run_time_binding(capsys):
+    """``examples/ablation_fixed_binding.py`` on C3 at full size: the library whose tile counts
+    were frozen for the benchmark batch and the run-time-bound one give identical bits on that
+    batch, on shorter batches and on batches with longer bags; every time is positive."""
+    import json
+    import sys
+    from recflex_amd import prebuilt
+    for name in ("c3_tuned", "c3_tuned_static"):
+        if not os.path.exists(prebuilt.lib_path(name)):
+            raise RuntimeError(f"{name} is not built: run __graft_entry__.build() first")
+    spec = importlib.util.spec_from_file_location(
+        "ablation_fixed_binding", os.path.join(ROOT, "examples", "ablation_fixed_binding.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    print("[case] examples/ablation_fixed_binding.py --workload c3 --steps 3", flush=True)
+    argv = sys.argv
+    sys.argv = ["ablation_fixed_binding.py", "--workload", "c3", "--steps", "3"]
+    try:
+        mod.main()
+    finally:
+        sys.argv = argv
+    summary = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert len(summary["cases"]) >= 8
+    for case in summary["cases"]:
+        assert case["identical_bits"], case["batch"]
+        assert case["run_time_binding_us"] > 0 and case["frozen_binding_us"] > 0
