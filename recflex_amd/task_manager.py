@@ -1,54 +1,92 @@
-"""Pool of worker processes gated by a queue of resources (GPU ids, compile slots).
+"""Runs tasks in child processes, at most one at a time per resource (a GPU id, a compile slot).
 
-Same interface and behaviour as ``RecFlex/task_manager.py:19-53``: ``add_task`` starts a thread
-that takes one resource from the queue, runs the target in a spawned process (passing the
-resource as keyword ``ident_key`` if given), waits for it and puts the resource back even if
-starting the process fails; ``join`` waits for all threads; more than ``max_threads``
-outstanding tasks force a join.  Added: the exit codes of the child processes are kept in
-``exit_codes`` so that a caller can tell a crashed worker from a finished one.
+The interface of ``RecFlex/task_manager.py:19-53``: ``TaskManager(resources, max_threads)``,
+``add_task(target, args, ident_key)`` -- run ``target(*args)`` in a spawned process, with the
+resource it was given as keyword ``ident_key`` if that is set -- and ``join()``.  The structure
+is another one: every resource has a serving thread that takes tasks from one shared queue for
+as long as there are any, so a thousand tasks cost as many processes but only ``len(resources)``
+threads, and a resource can never be handed to two tasks.  ``join`` waits until the queue has
+drained and the serving threads have ended; the next ``add_task`` starts them again.  More than
+``max_threads`` unfinished tasks make ``add_task`` wait for all of them first, as in the reference.
+Added: ``exit_codes`` keeps the exit code of every child (``None`` if it could not be started), so
+that a caller can tell a crashed worker from a finished one.
 """
 
 import multiprocessing as mp
 import queue
 import threading
-from typing import Any, List
+from typing import Any, Callable, List, Optional, Sequence, Tuple
+
+_Task = Tuple[Callable, Sequence[Any], Optional[str]]
 
 
 class TaskManager:
     def __init__(self, resources: List[Any], max_threads: int = 256):
-        self.resource_queue = queue.Queue(len(resources))
-        for resource in resources:
-            self.resource_queue.put(resource)
-        self.task_threads: List[threading.Thread] = []
-        self.max_threads = max_threads
-        self.exit_codes: List[int] = []
-        self._lock = threading.Lock()
-
         assert mp.get_start_method() == 'spawn', \
             "Please add multiprocessing.set_start_method('spawn') at the start of your program!"
+        self.resources: List[Any] = list(resources)
+        self.max_threads = max_threads
+        self.exit_codes: List[Optional[int]] = []
+        self._tasks: "queue.Queue[Optional[_Task]]" = queue.Queue()
+        self._servers: List[threading.Thread] = []
+        self._busy: List[Any] = []
+        self._lock = threading.Lock()
 
-    def _exec(self, target, args, ident_key: str = None):
-        ident = self.resource_queue.get()
-        try:
-            kwargs = {ident_key: ident} if ident_key else {}
-            p = mp.Process(target=target, args=args, kwargs=kwargs)
-            p.start()
-            p.join()
+    # ---- one serving thread per resource --------------------------------------------------
+
+    def _serve(self, resource: Any) -> None:
+        while True:
+            task = self._tasks.get()
+            if task is None:                    # join() is over: nothing more will come
+                self._tasks.task_done()
+                return
+            target, args, ident_key = task
+            code: Optional[int] = None
             with self._lock:
-                self.exit_codes.append(p.exitcode)
-        finally:
-            self.resource_queue.put(ident)
+                self._busy.append(resource)
+            try:
+                child = mp.Process(target=target, args=tuple(args),
+                                   kwargs={ident_key: resource} if ident_key else {})
+                child.start()
+                child.join()
+                code = child.exitcode
+            finally:
+                with self._lock:
+                    self._busy.remove(resource)
+                    self.exit_codes.append(code)
+                self._tasks.task_done()
 
-    def add_task(self, target, args, ident_key: str = None):
-        thread = threading.Thread(target=self._exec, args=(target, args, ident_key))
-        self.task_threads.append(thread)
-        thread.start()
+    def _start_servers(self) -> None:
+        if not self._servers:
+            self._servers = [threading.Thread(target=self._serve, args=(r,), daemon=True)
+                             for r in self.resources]
+            for server in self._servers:
+                server.start()
 
-        if len(self.task_threads) >= self.max_threads:
-            print("Too many tasks have been added! Forced to wait for previous threads finishing.")
+    # ---- the reference's interface --------------------------------------------------------
+
+    def add_task(self, target: Callable, args: Sequence[Any], ident_key: str = None) -> None:
+        if self._tasks.unfinished_tasks >= self.max_threads:
+            print("Too many tasks have been added! Forced to wait for previous tasks finishing.")
             self.join()
+        self._start_servers()
+        self._tasks.put((target, args, ident_key))
 
-    def join(self):
-        for thread in self.task_threads:
-            thread.join()
-        self.task_threads = []
+    def join(self) -> None:
+        """Returns when every task added so far has run."""
+        self._tasks.join()
+        for _ in self._servers:
+            self._tasks.put(None)
+        for server in self._servers:
+            server.join()
+        self._servers = []
+
+    @property
+    def resource_queue(self) -> "queue.Queue[Any]":
+        """The resources no task holds right now (a snapshot, in the reference's form)."""
+        with self._lock:
+            idle = [r for r in self.resources if r not in self._busy]
+        snapshot: "queue.Queue[Any]" = queue.Queue(len(self.resources))
+        for resource in idle:
+            snapshot.put(resource)
+        return snapshot
