@@ -22,6 +22,7 @@ CDNA4 specifics: occupancy is counted in 256-thread workgroups per CU (= wavefro
 are compiled once and shared through ``.cache/``.
 """
 
+import filecmp
 import hashlib
 import json
 import os
@@ -294,6 +295,22 @@ class Tuner:
             self._headers_digest_cache = h.digest()
         return self._headers_digest_cache
 
+    def _kept(self, output_dir: str, tune_config: TuneConfig) -> bool:
+        """The resume-by-files rule (RecFlex/tuning/tuner.py:117): an existing library is kept --
+        if it is what this directory's source gives under the device headers as they are now.  A
+        library left by a run with older headers would load (or be refused for its ABI version)
+        long after the compile step that should have replaced it."""
+        lib = f"{output_dir}/build/librecom.so"
+        if tune_config.recompile or not os.path.exists(lib):
+            return False
+        if not os.path.exists(f"{output_dir}/process.hip"):
+            return False
+        cached = self._cached_lib(self._source_key(output_dir))
+        if not os.path.exists(cached):
+            return False
+        # the same file (a hard link), or a copy of it (where links are refused or were not kept)
+        return os.path.samefile(lib, cached) or filecmp.cmp(lib, cached, shallow=False)
+
     def _cached_lib(self, key: str) -> str:
         return f"{self.basic.codegen_dir}/.cache/{key}/librecom.so"
 
@@ -362,7 +379,7 @@ class Tuner:
         for feat_id in range(self.num_feats):
             for occupancy in tune_config.occupancies:
                 output_dir, build_dir = self.get_output_build_dir(feat_id, occupancy)
-                if not os.path.exists(f"{build_dir}/librecom.so") or tune_config.recompile:
+                if not self._kept(output_dir, tune_config):
                     os.makedirs(build_dir, exist_ok=True)
                     padded = self.pad_sched_params(self.feat_sched_param_candidates[feat_id],
                                                    self.local_padded_num(feat_id, occupancy, tune_config))
@@ -461,7 +478,7 @@ class Tuner:
         jobs = []
         for occupancy in tune_config.occupancies:
             output_dir, build_dir = self.get_tournament_dir(occupancy)
-            if not os.path.exists(f"{build_dir}/librecom.so") or tune_config.recompile:
+            if not self._kept(output_dir, tune_config):
                 os.makedirs(build_dir, exist_ok=True)
                 admitted = self.tournament_candidates(occupancy, tune_config)
                 with open(f"{output_dir}/admitted.json", "w") as f:
@@ -663,7 +680,7 @@ class Tuner:
                     timing: bool = False) -> bool:
         """Emit a whole-model kernel if its library is missing; True if a build is needed."""
         build_dir = f"{output_dir}/build"
-        if os.path.exists(f"{build_dir}/librecom.so") and not tune_config.recompile:
+        if self._kept(output_dir, tune_config):
             return False
         os.makedirs(build_dir, exist_ok=True)
         self.emit_codes(output_dir=output_dir, feat_schedules=sched_params, occupancy=occupancy,
@@ -942,7 +959,7 @@ class Tuner:
         for feat_id in range(self.num_feats):
             for sched_param_id, sched_param in enumerate(self.feat_sched_param_candidates[feat_id]):
                 output_dir, build_dir = get_output_build_dir(feat_id, sched_param_id)
-                if not os.path.exists(f"{build_dir}/librecom.so") or tune_config.recompile:
+                if not self._kept(output_dir, tune_config):
                     os.makedirs(build_dir, exist_ok=True)
                     self.emit_codes(output_dir=output_dir, feat_schedules=[sched_param], occupancy=None,
                                     inline=tune_config.inline, timing=False, tune=False,

@@ -393,3 +393,32 @@ def test_whole_passes_when_tiles_are_plentiful():
     assert tiles_per_feature(*args, grid_blocks=1280)[0] == 512  # 512 * 100 >= 2 * 1280
     few = ([off[:33]] * 4, [516] * 4, [516] * 4, [4] * 4, 65536)
     assert tiles_per_feature(*few, grid_blocks=1280)[0] == 32    # 8 * 4 < 2 * 1280: spread out
+
+
+def test_an_existing_library_is_kept_only_if_it_is_the_build_of_todays_sources(tmp_path, monkeypatch):
+    """The resume-by-files rule keeps ``build/librecom.so`` when it is the cache entry of the
+    directory's ``process.hip`` under the current device headers -- and rebuilds otherwise."""
+    t = _tiny_tuner(tmp_path)
+    cfg = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=2, in_process=True)
+    out = str(tmp_path / "some" / "o4")
+    os.makedirs(f"{out}/build")
+    assert not t._kept(out, cfg)                                 # nothing there
+    with open(f"{out}/process.hip", "w") as f:
+        f.write("// source\n")
+    with open(f"{out}/build/librecom.so", "wb") as f:
+        f.write(b"library bytes")
+    assert not t._kept(out, cfg)                                 # a library nobody vouches for
+    cached = t._cached_lib(t._source_key(out))
+    os.makedirs(os.path.dirname(cached))
+    with open(cached, "wb") as f:
+        f.write(b"library bytes")
+    assert t._kept(out, cfg)                                     # a copy of the cache entry
+    assert not t._kept(out, cfg._replace(recompile=True))
+    with open(f"{out}/build/librecom.so", "wb") as f:
+        f.write(b"other bytes..")                                # same size, other content
+    assert not t._kept(out, cfg)
+    os.remove(f"{out}/build/librecom.so")
+    os.link(cached, f"{out}/build/librecom.so")
+    assert t._kept(out, cfg)                                     # the cache entry itself
+    monkeypatch.setattr(t, "_headers_digest", lambda: b"headers edited since")
+    assert not t._kept(out, cfg)                                 # built under other headers
