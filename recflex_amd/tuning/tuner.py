@@ -304,7 +304,7 @@ class Tuner:
         if tune_config.recompile or not os.path.exists(lib):
             return False
         if not os.path.exists(f"{output_dir}/process.hip"):
-            return False
+            return True         # nothing to hold it against: the reference's rule as it is
         cached = self._cached_lib(self._source_key(output_dir))
         if not os.path.exists(cached):
             return False

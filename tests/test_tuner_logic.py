@@ -403,10 +403,11 @@ def test_an_existing_library_is_kept_only_if_it_is_the_build_of_todays_sources(t
     out = str(tmp_path / "some" / "o4")
     os.makedirs(f"{out}/build")
     assert not t._kept(out, cfg)                                 # nothing there
-    with open(f"{out}/process.hip", "w") as f:
-        f.write("// source\n")
     with open(f"{out}/build/librecom.so", "wb") as f:
         f.write(b"library bytes")
+    assert t._kept(out, cfg)                                     # no source to hold it against
+    with open(f"{out}/process.hip", "w") as f:
+        f.write("// source\n")
     assert not t._kept(out, cfg)                                 # a library nobody vouches for
     cached = t._cached_lib(t._source_key(out))
     os.makedirs(os.path.dirname(cached))
