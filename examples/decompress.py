@@ -5,7 +5,8 @@
 ``compress/A/feat_map.txt`` (written by ``compress.py``) says which original features each
 representative stands for; the per-feature result directories ``output/f{k}`` of the compressed
 model (``output/naive/f{k}`` with ``--naive``) are copied to ``output/f{j}`` of the full model for
-every ``j`` in cluster ``k``.  A following ``tune.py -m models/A --interference replicate`` finds
+every ``j`` in cluster ``k``, and the compressed model's compile cache (``output/.cache``) with
+them.  A following ``tune.py -m models/A --interference replicate`` finds
 the libraries and measurements there and goes straight to the global stage.
 
 Same command line and behaviour as the reference's ``examples/decompress.py:14-54``.  (The
@@ -35,6 +36,11 @@ def restore_output(src_root: str, dst_root: str, clusters: List[List[int]]) -> i
         for feat_id in members:
             shutil.copytree(src, os.path.join(dst_root, f"f{feat_id}"), dirs_exist_ok=True)
             copied += 1
+    # the compile cache goes along: the full model's tuner keeps a library it finds only if the
+    # cache holds the build of that directory's source under the current device headers
+    cache = os.path.join(src_root, ".cache")
+    if os.path.isdir(cache):
+        shutil.copytree(cache, os.path.join(dst_root, ".cache"), dirs_exist_ok=True)
     return copied
 
 
