@@ -8,8 +8,8 @@ key over the model's emitted source and the device headers, and a library built 
 else gets ``None``.
 
     python -m recflex_amd.hbm_traffic record --model c3_tuned \\
-        --fetch-csv gpurun_out/pmc_fetch_c3/x_counter_collection.csv \\
-        --write-csv gpurun_out/pmc_write_c3/x_counter_collection.csv --copy-bytes 805306368
+        --fetch-csv prof/pmc_fetch_c3/x_counter_collection.csv \\
+        --write-csv prof/pmc_write_c3/x_counter_collection.csv --copy-bytes 805306368
 
 ``FETCH_SIZE`` / ``WRITE_SIZE`` are what the L2 caches exchange with the memory side, in units
 that a plain copy of known size calibrates: the runs hold one device-to-device copy of
