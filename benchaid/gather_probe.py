@@ -1,10 +1,10 @@
-"""Gather probe: time the bare fetch of the rows a batch looks up (``csrc/probe/gather_probe.hip``).
+"""Gather probe: time the bare fetch of the rows a batch looks up (``csrc/gather_probe.hip``).
 
 Measurement aid for ``bench.py``: the same tables and index streams as the fused kernel, 16-byte
 loads, no sums and no output, swept over the loads in flight per lane, the resident workgroups
-per CU, the bytes per chunk and the XCD-segmented walk; the fastest setting is reported.  Its time is
-what the memory system (HBM, Infinity Cache, L2, L1 miss handling) needs for the rows of this
-batch alone.
+per CU, the bytes per chunk and the XCD-segmented walk; the fastest setting is reported.  Its
+time is an empirical reference -- another kernel that fetches the same rows and does nothing
+else -- not a bound: the fused kernel has been faster than it on some batches.
 """
 
 import ctypes
@@ -23,8 +23,11 @@ SWEEP_SEGMENTS = (0, 16, 32)
 SWEEP_CHUNK_BYTES = (16384, 65536)
 
 
+AID_DIR = os.path.dirname(os.path.abspath(__file__))
+
+
 def lib_path() -> str:
-    return os.path.join(BasicBuilder().csrc_dir, "build", "libgather_probe.so")
+    return os.path.join(AID_DIR, "build", "libgather_probe.so")
 
 
 def build(force: bool = False) -> str:
@@ -32,7 +35,7 @@ def build(force: bool = False) -> str:
     lib = lib_path()
     if force or not os.path.exists(lib):
         os.makedirs(os.path.dirname(lib), exist_ok=True)
-        src = os.path.join(basic.csrc_dir, "probe", "gather_probe.hip")
+        src = os.path.join(AID_DIR, "csrc", "gather_probe.hip")
         tmp = lib + f".tmp{os.getpid()}"
         subprocess.run([basic.hipcc, *basic.hip_flags, "-O3", src, "-o", tmp], check=True)
         os.replace(tmp, lib)
@@ -61,7 +64,7 @@ def calibration_copy(nbytes: int, device="cuda:0") -> None:
     import torch
     path = lib_path()
     if not os.path.exists(path):
-        raise FileNotFoundError(f"{path} is missing: build it with recflex_amd.gather_probe.build()")
+        raise FileNotFoundError(f"{path} is missing: build it with benchaid.gather_probe.build()")
     lib = ctypes.CDLL(path)
     lib.calibration_copy_launch.restype = ctypes.c_int
     lib.calibration_copy_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
@@ -87,7 +90,7 @@ class GatherProbe:
         import torch
         path = lib_path()
         if not os.path.exists(path):
-            raise FileNotFoundError(f"{path} is missing: build it with recflex_amd.gather_probe.build()")
+            raise FileNotFoundError(f"{path} is missing: build it with benchaid.gather_probe.build()")
         self.lib = ctypes.CDLL(path)
         self.lib.gather_probe_launch.restype = ctypes.c_int
         self.lib.gather_probe_launch.argtypes = [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 5 + \

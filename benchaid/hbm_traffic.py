@@ -2,12 +2,12 @@
 
 A live benchmark run cannot read the memory counters; ``rocprofv3 --pmc FETCH_SIZE`` and
 ``--pmc WRITE_SIZE`` runs of ``bench.py`` can.  This module turns the two counter files of such
-runs into one record per model in ``recflex_amd/tuned/hbm_traffic.json`` and hands the figure
+runs into one record per model in ``benchaid/hbm_traffic.json`` and hands the figure
 back to ``bench.py`` -- but only for the very library it was measured on: every record carries a
 key over the model's emitted source and the device headers, and a library built from anything
 else gets ``None``.
 
-    python -m recflex_amd.hbm_traffic record --model c3_tuned \\
+    python -m benchaid.hbm_traffic record --model c3_tuned \\
         --fetch-csv prof/pmc_fetch_c3/x_counter_collection.csv \\
         --write-csv prof/pmc_write_c3/x_counter_collection.csv --copy-bytes 805306368
 
@@ -26,12 +26,12 @@ import json
 import os
 from typing import Dict, List, Optional, Tuple
 
-from .code_emitter.build_basic import BasicBuilder
-from . import prebuilt
+from recflex_amd.code_emitter.build_basic import BasicBuilder
+from recflex_amd import prebuilt
 
 CALIBRATION_KERNEL = "CalibrationCopyKnl"      # launched by gather_probe.calibration_copy
 
-RECORD_PATH = os.path.join(prebuilt.TUNED_DIR, "hbm_traffic.json")
+RECORD_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "hbm_traffic.json")
 
 
 def library_key(model: str) -> Optional[str]:
@@ -56,13 +56,22 @@ def load_records() -> Dict[str, dict]:
         return json.load(f)
 
 
-def recorded_traffic_bytes(model: str) -> Optional[float]:
-    """HBM bytes per launch of ``FusedKnl`` of this model, if counters were taken on the library
-    as it is built now; ``None`` otherwise."""
+def recorded_traffic(model: str) -> Optional[dict]:
+    """Memory-side bytes per launch of ``FusedKnl`` of this model (``bytes``, ``read_bytes``,
+    ``written_bytes``, ``source``), if counters were taken on the library as it is built now;
+    ``None`` otherwise."""
     rec = load_records().get(model)
     if not rec or rec.get("key") != library_key(model):
         return None
-    return float(rec["bytes"])
+    return {"bytes": float(rec["bytes"]), "read_bytes": float(rec["read_bytes"]),
+            "written_bytes": float(rec["written_bytes"]),
+            "source": "recorded in benchaid/hbm_traffic.json for this library (key over its emitted "
+                      "source and the device headers)" + (": " + rec["note"] if rec.get("note") else "")}
+
+
+def recorded_traffic_bytes(model: str) -> Optional[float]:
+    rec = recorded_traffic(model)
+    return rec["bytes"] if rec else None
 
 
 def _counter_files(path: str) -> List[str]:
@@ -84,9 +93,11 @@ def read_counter(path: str, counter: str) -> Dict[str, List[float]]:
     return out
 
 
-def _fused_and_copy(readings: Dict[str, List[float]], copy_substr: str) -> Tuple[float, int, float]:
-    """(mean reading of FusedKnl, its dispatches, reading of the one calibration copy)."""
-    fused = readings.get("FusedKnl")
+def _fused_and_copy(readings: Dict[str, List[float]], copy_substr: str,
+                    skip_first: int = 0) -> Tuple[float, int, float]:
+    """(mean reading of FusedKnl after its first ``skip_first`` dispatches, the dispatches that
+    count, reading of the one calibration copy)."""
+    fused = (readings.get("FusedKnl") or [])[skip_first:]
     if not fused:
         raise ValueError("the counter file holds no FusedKnl dispatch")
     copies = [v for name, vals in readings.items() if copy_substr in name for v in vals]
@@ -97,17 +108,17 @@ def _fused_and_copy(readings: Dict[str, List[float]], copy_substr: str) -> Tuple
     return sum(fused) / len(fused), len(fused), copies[0]
 
 
-def record(model: str, fetch_csv: str, write_csv: str, copy_bytes: int,
-           copy_substr: str = CALIBRATION_KERNEL) -> dict:
-    key = library_key(model)
-    if key is None:
-        raise FileNotFoundError(f"{prebuilt.model_dir(model)}/process.hip: build the model first")
-    fetch, n_fetch, copy_fetch = _fused_and_copy(read_counter(fetch_csv, "FETCH_SIZE"), copy_substr)
-    write, n_write, copy_write = _fused_and_copy(read_counter(write_csv, "WRITE_SIZE"), copy_substr)
+def traffic_from_counter_files(fetch_csv: str, write_csv: str, copy_bytes: int,
+                               copy_substr: str = CALIBRATION_KERNEL, skip_first: int = 0) -> dict:
+    """Bytes per launch of FusedKnl from a FETCH_SIZE and a WRITE_SIZE run (files or directories
+    of rocprofv3 ``--pmc`` csv output), each counter scaled by its reading for the calibration
+    copy of ``copy_bytes`` bytes in the same run; the first ``skip_first`` FusedKnl dispatches of
+    each run (warm-up launches) are left out of the mean."""
+    fetch, n_fetch, copy_fetch = _fused_and_copy(read_counter(fetch_csv, "FETCH_SIZE"), copy_substr, skip_first)
+    write, n_write, copy_write = _fused_and_copy(read_counter(write_csv, "WRITE_SIZE"), copy_substr, skip_first)
     fetch_factor = copy_bytes / copy_fetch          # bytes per counter unit
     write_factor = copy_bytes / copy_write
-    rec = {
-        "key": key,
+    return {
         "fetch_reading": fetch, "write_reading": write,
         "fetch_bytes_per_unit": fetch_factor, "write_bytes_per_unit": write_factor,
         "read_bytes": fetch * fetch_factor, "written_bytes": write * write_factor,
@@ -115,6 +126,16 @@ def record(model: str, fetch_csv: str, write_csv: str, copy_bytes: int,
         "dispatches": [n_fetch, n_write],
         "calibration": f"the {copy_substr} dispatch = a copy of {copy_bytes} bytes",
     }
+
+
+def record(model: str, fetch_csv: str, write_csv: str, copy_bytes: int,
+           copy_substr: str = CALIBRATION_KERNEL, skip_first: int = 0, note: str = "") -> dict:
+    key = library_key(model)
+    if key is None:
+        raise FileNotFoundError(f"{prebuilt.model_dir(model)}/process.hip: build the model first")
+    rec = dict(traffic_from_counter_files(fetch_csv, write_csv, copy_bytes, copy_substr, skip_first), key=key)
+    if note:
+        rec["note"] = note
     records = load_records()
     records[model] = rec
     with open(RECORD_PATH, "w") as f:
@@ -131,11 +152,13 @@ def main() -> None:
     rec.add_argument("--write-csv", required=True)
     rec.add_argument("--copy-bytes", type=int, required=True)
     rec.add_argument("--copy-kernel", default=CALIBRATION_KERNEL, help="substring of the copy kernel's name")
+    rec.add_argument("--skip-first", type=int, default=0, help="FusedKnl dispatches to leave out (warm-up)")
+    rec.add_argument("--note", default="", help="how the runs were made, kept with the record")
     sub.add_parser("show", help="print the records and whether each matches the library as built now")
     args = parser.parse_args()
     if args.cmd == "record":
         print(json.dumps(record(args.model, args.fetch_csv, args.write_csv, args.copy_bytes,
-                                args.copy_kernel), indent=1))
+                                args.copy_kernel, args.skip_first, args.note), indent=1))
     else:
         for model, r in load_records().items():
             print(f"{model}: {r['bytes'] / 1e6:.1f} MB per launch "

@@ -8,7 +8,8 @@ Flags as in the reference's ``examples/tune.py:35-51``.  ``-m`` names a model di
 ``table_config.txt``, ``schedule_config.txt`` and ``data/`` (``batch_sizes.txt`` + ``f{i}.txt``).
 Additions: ``--workload c3`` tunes one of the built-in synthetic configurations instead of a
 model directory; ``--compile_only`` stops after emitting and building the local-stage kernels
-(no GPU needed -- a later run finds the libraries and only measures); ``--occupancies`` and
+and the default-schedule contenders of the global stage (no GPU needed -- a later run finds
+the libraries, measures, and builds only the mix it elects); ``--occupancies`` and
 ``--sample_batch_nums`` bound the search; ``--profiler events`` times the global stage with
 events instead of spawning rocprofv3.  The result is ``<output>/optimal/`` (sources, library,
 ``schedule.json``).
@@ -189,6 +190,8 @@ def main():
             tuner.compile_tournament(tune_config)
         else:
             tuner.compile_local(tune_config)
+        # ... and the contenders of the global stage that are known without a measurement
+        tuner.compile_default_contenders(tune_config)
         print(f"local-stage kernels built under {tuner.basic.codegen_dir}")
         return
 

@@ -34,6 +34,9 @@ its library is missing.  Names:
                    ``fewbags_unsplit``: the same with one workgroup per bag, for comparison
 ``manysplit``      17 fp16 features of dim 256 under the split-bag schedule: 36 MB of workspace,
                    more than the static array of ``recom_process_static_workspace`` may hold
+``refa``, ``reff4`` models shaped like the reference's example models A and a quarter of F (1 000 and
+                   2 500 small features, batch 256; ``workloads.REF_SHAPED``), default schedules;
+                   ``refa_tuned``: with ``tuned/refa_schedule.json`` if that file exists
 ``wide``           1 500 small features (several binding rounds per thread)
 ``wider``          2 500 small features (bound once per launch by the binding kernel)
 """
@@ -294,6 +297,10 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "manysplit": _many_split,
     "wide": _wide,
     "wider": lambda: _wide(2500, "wider"),
+    # models shaped like the reference's own examples (workloads.REF_SHAPED), default schedules
+    "refa": lambda: _default(make_workload("REFA")),
+    "reff4": lambda: _default(make_workload("REFF4")),
+    "refa_tuned": lambda: _tuned(make_workload("REFA"), "refa_schedule.json"),
     "b128": lambda: _other_block_size(128),
     "b512": lambda: _other_block_size(512),
 }
@@ -501,4 +508,34 @@ def build_compress_fixture(model_dir: str) -> str:
                    stdout=subprocess.DEVNULL)
     tuner = make_fixture_tuner(small, codegen_dir=os.path.join(small, "output"))
     tuner.compile_local(fixture_tune_config(recompile=True, interference="replicate", occupancies=[4]))
+    return root
+
+
+# ------------------------------------------------------------------------------------------------
+# the two command-line entry points run end to end (examples/tune.py -m ..., then
+# examples/test.py -m ... -o .../optimal --check): everything tune.py can compile before it has
+# measured anything is built ahead, so a GPU machine only measures and builds the mix it elects
+# ------------------------------------------------------------------------------------------------
+
+ENTRY_TUNE_FLAGS = ["--occupancies", "4", "--sample_batch_nums", "2", "-n", "4"]
+
+
+def entry_fixture_dir() -> str:
+    return os.path.join(MODELS_DIR, "tune_entry")
+
+
+def build_entry_point_fixture(model_dir: str) -> str:
+    """``tune_entry/model``: a copy of the fixture model directory with ``output/`` as
+    ``examples/tune.py -m tune_entry/model --compile_only`` leaves it (tournament kernel and
+    default-schedule contender at the occupancy of ``ENTRY_TUNE_FLAGS``)."""
+    import shutil
+    import subprocess
+    import sys
+    root = entry_fixture_dir()
+    shutil.rmtree(root, ignore_errors=True)
+    model = os.path.join(root, "model")
+    shutil.copytree(model_dir, model)
+    script = os.path.join(os.path.dirname(PACKAGE_DIR), "examples", "tune.py")
+    subprocess.run([sys.executable, script, "-m", model, "--compile_only", "--recompile", *ENTRY_TUNE_FLAGS],
+                   check=True, stdout=subprocess.DEVNULL)
     return root

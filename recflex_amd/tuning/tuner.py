@@ -735,17 +735,31 @@ class Tuner:
             return None      # rocprof_profile spawns its own process; run them one after another
         return TaskManager(tune_config.gpu_ids[0:1])
 
+    def default_contenders(self, tune_config: TuneConfig) -> list:
+        """(directory, occupancy, schedules) of the default-heuristic mix at every occupancy: the
+        contenders of the global stage that are known before anything is measured."""
+        if not tune_config.include_default:
+            return []
+        default_mix = [self.feat_sched_param_candidates[f][k]
+                       for f, k in enumerate(self.default_choices()[0])]
+        return [(f"{self.basic.codegen_dir}/default/o{occupancy}", occupancy, default_mix)
+                for occupancy in tune_config.occupancies]
+
+    def compile_default_contenders(self, tune_config: TuneConfig) -> None:
+        """Emit and build ``default/o{occ}`` (no GPU needed)."""
+        jobs = []
+        for output_dir, occupancy, sched_params in self.default_contenders(tune_config):
+            if self._build_full(output_dir, sched_params, occupancy, tune_config):
+                jobs.append((output_dir, f"{output_dir}/build"))
+        self._schedule_builds(jobs, tune_config)
+
     def tune_occupancy(self, occu_opt_sched_params: List[List[Tuple[ScheduleBase, NamedTuple]]],
                        tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
         # contenders: (directory, occupancy, schedules)
         contenders = []
         for occupancy, sched_params in zip(tune_config.occupancies, occu_opt_sched_params):
             contenders.append((self.get_output_build_dir(-1, occupancy)[0], occupancy, sched_params))
-        if tune_config.include_default:
-            default_mix = [self.feat_sched_param_candidates[f][k]
-                           for f, k in enumerate(self.default_choices()[0])]
-            for occupancy in tune_config.occupancies:
-                contenders.append((f"{self.basic.codegen_dir}/default/o{occupancy}", occupancy, default_mix))
+        contenders += self.default_contenders(tune_config)
 
         jobs = []
         for output_dir, occupancy, sched_params in contenders:

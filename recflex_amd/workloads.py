@@ -44,6 +44,11 @@ class FeatureSpec(NamedTuple):
     # > 0: bag lengths from a lognormal of mean mean_bag and this sigma of the logarithm instead
     # of a Poisson (a heavy tail: at 1.5 the longest of 2 048 bags is some hundred means long)
     len_sigma: float = 0.0
+    # > 0: bag lengths from N(mean_bag, len_std) restricted to [0, len_max] (len_max 0 = no upper
+    # end) and truncated to integers: the "multi-hot" families of the reference's data generator
+    # (data_synthesis/data_generate.py:27-40)
+    len_std: float = 0.0
+    len_max: int = 0
 
 
 class Workload(NamedTuple):
@@ -87,13 +92,77 @@ def _log_uniform(rng: np.random.Generator, lo: float, hi: float, n: int) -> np.n
     return np.exp(rng.uniform(math.log(lo), math.log(hi), n))
 
 
+# Models shaped like the reference's own example models (examples/models/A .. F there: 800 to
+# 10 000 features, tables of 1 024 to 16 384 rows, dims 4 to 128, batches of at most 512): half
+# the features one-hot, the rest "multi-hot" (truncated normal pooling factor), "multi-hot-static"
+# (fixed pooling factor) and "multi-hot-one-side" (normal truncated at 0 only), in groups of like
+# features.  Only these shape parameters are taken from there; every group's parameters, every
+# table shape and every index is drawn here from the seed.
+REF_SHAPED = {
+    # name: (features, batch, seed, share of one-hot / multi-hot / static / one-side features)
+    "REFA": (1000, 256, 2001, (0.50, 0.25, 0.15, 0.10)),
+    "REFF4": (2500, 256, 2002, (0.50, 0.35, 0.15, 0.0)),
+}
+REF_GROUP = 50            # like features per group
+REF_ZIPF_ALPHA = 1.05
+
+
+def _table_rules():
+    """TABLE_RULES / DIM_CHOICES of data_synthesis/table_config_generate.py (rows and the weighted
+    choice of dims per feature family), loaded from that script."""
+    import os
+    from .utils import import_from_path
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    mod = import_from_path("table_config_generate",
+                           os.path.join(root, "data_synthesis", "table_config_generate.py"))
+    return mod.TABLE_RULES, mod.DIM_CHOICES
+
+
+def make_ref_shaped(name: str, batch: Optional[int] = None, num_features: Optional[int] = None,
+                    seed: Optional[int] = None) -> Workload:
+    import random
+    total, B, base_seed, shares = REF_SHAPED[name]
+    total = num_features or total
+    B = batch or B
+    seed = base_seed if seed is None else seed
+    rules, dim_choices = _table_rules()
+    rng = np.random.default_rng(seed)
+    dims_rng = random.Random(seed)
+    kinds = ("one-hot", "multi-hot", "multi-hot-static", "multi-hot-one-side")
+    counts = [int(round(total * share)) for share in shares]
+    last = max(k for k, share in enumerate(shares) if share > 0)
+    counts[last] = total - sum(c for k, c in enumerate(counts) if k != last)   # rounding
+    feats: List[FeatureSpec] = []
+    for kind, count in zip(kinds, counts):
+        rows, weights = rules[kind]
+        for g0 in range(0, count, REF_GROUP):
+            n = min(REF_GROUP, count - g0)
+            coverage = float(rng.choice([0.3, 0.5, 0.8, 1.0])) if kind != "one-hot" else 1.0
+            mean = float(rng.choice([10, 50, 100, 200] if kind == "multi-hot-one-side" else [10, 50, 100]))
+            std = mean * float(rng.choice([0.2, 0.5, 1.0]))
+            top = int(mean * float(rng.choice([2, 5])))
+            for dim in dims_rng.choices(dim_choices, weights, k=n):
+                if kind == "one-hot":
+                    spec = FeatureSpec(rows, dim, "float", 1.0, True, 1.0 - coverage, REF_ZIPF_ALPHA)
+                elif kind == "multi-hot-static":
+                    spec = FeatureSpec(rows, dim, "float", mean, True, 1.0 - coverage, REF_ZIPF_ALPHA)
+                else:
+                    spec = FeatureSpec(rows, dim, "float", mean, False, 1.0 - coverage, REF_ZIPF_ALPHA,
+                                       len_std=std, len_max=top if kind == "multi-hot" else 0)
+                feats.append(spec)
+    return Workload(name, B, seed, tuple(feats))
+
+
 def make_workload(name: str, batch: Optional[int] = None, num_features: Optional[int] = None,
                   max_rows: Optional[int] = None, seed: Optional[int] = None) -> Workload:
-    """One of C1..C5.  ``batch`` / ``num_features`` / ``max_rows`` shrink the configuration
-    (same distributions, smaller extents) for tests that must run in seconds."""
+    """One of C1..C5, or one of the reference-shaped models REFA / REFF4.  ``batch`` /
+    ``num_features`` / ``max_rows`` shrink the configuration (same distributions, smaller
+    extents) for tests that must run in seconds."""
     name = name.upper()
+    if name in REF_SHAPED:
+        return make_ref_shaped(name, batch, num_features, seed)
     if name not in BASE_SEEDS:
-        raise ValueError(f"unknown workload {name!r}; expected one of {sorted(BASE_SEEDS)}")
+        raise ValueError(f"unknown workload {name!r}; expected one of {sorted(BASE_SEEDS) + sorted(REF_SHAPED)}")
     seed = BASE_SEEDS[name] if seed is None else seed
     rng = np.random.default_rng(seed)
 
@@ -168,6 +237,16 @@ def gen_feature_inputs(spec: FeatureSpec, batch: int, seed_seq: np.random.SeedSe
     rng = np.random.Generator(np.random.PCG64(seed_seq))
     if spec.fixed_len:
         lens = np.full(batch, int(round(spec.mean_bag)), dtype=np.int64)
+    elif spec.len_std > 0:
+        hi = float(spec.len_max) if spec.len_max > 0 else np.inf
+        lens = np.empty(batch, dtype=np.int64)
+        filled = 0
+        while filled < batch:               # rejection sampling of the truncated normal
+            draw = rng.normal(spec.mean_bag, spec.len_std, max(2 * (batch - filled), 16))
+            draw = draw[(draw >= 0) & (draw <= hi)]
+            take = min(len(draw), batch - filled)
+            lens[filled:filled + take] = draw[:take].astype(np.int64)
+            filled += take
     elif spec.len_sigma > 0:
         mu = np.log(max(spec.mean_bag, 0.05)) - spec.len_sigma ** 2 / 2
         lens = np.floor(rng.lognormal(mu, spec.len_sigma, batch) + rng.random(batch)).astype(np.int64)
@@ -189,14 +268,18 @@ def gen_feature_inputs(spec: FeatureSpec, batch: int, seed_seq: np.random.SeedSe
     return idx.astype(np.int32), offsets.astype(np.int32)
 
 
-def gen_inputs(wl: Workload) -> Tuple[List[np.ndarray], List[np.ndarray]]:
+def gen_inputs(wl: Workload, workers: int = 0) -> Tuple[List[np.ndarray], List[np.ndarray]]:
+    """Indices and offsets of every feature.  ``workers`` > 1 draws the features on that many
+    threads (each feature has its own child seed, so the result does not depend on it)."""
     children = np.random.SeedSequence(wl.seed).spawn(wl.num_features)
-    indices, offsets = [], []
-    for spec, child in zip(wl.features, children):
-        i, o = gen_feature_inputs(spec, wl.batch, child)
-        indices.append(i)
-        offsets.append(o)
-    return indices, offsets
+    if workers > 1 and wl.num_features > 1:
+        from concurrent.futures import ThreadPoolExecutor
+        with ThreadPoolExecutor(max_workers=workers) as pool:
+            pairs = list(pool.map(lambda sc: gen_feature_inputs(sc[0], wl.batch, sc[1]),
+                                  zip(wl.features, children)))
+    else:
+        pairs = [gen_feature_inputs(spec, wl.batch, child) for spec, child in zip(wl.features, children)]
+    return [p[0] for p in pairs], [p[1] for p in pairs]
 
 
 def _integer_rows(spec: FeatureSpec, g, device, n: int):

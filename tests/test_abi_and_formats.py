@@ -213,7 +213,7 @@ def test_rocprof_stats_reader(tmp_path):
 
 
 def test_gather_probe_chunks_cover_every_lookup_once():
-    from recflex_amd.gather_probe import make_chunks, CHUNK_LOOKUPS
+    from benchaid.gather_probe import make_chunks, CHUNK_LOOKUPS
     lookups = [2500, 0, 10, 1024]
     vectors = [2, 9, 64, 1]
     chunks = make_chunks(lookups, vectors)

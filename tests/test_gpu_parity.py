@@ -223,7 +223,7 @@ def test_gather_probe_runs():
     run to completion on ragged inputs (empty features, rows of 1 to 64 vectors) and take time."""
     import torch
     from recflex_amd import prebuilt
-    from recflex_amd.gather_probe import GatherProbe
+    from benchaid.gather_probe import GatherProbe
     from recflex_amd.workloads import gen_inputs, gen_tables, row_stride
 
     wl = prebuilt.model_spec("edge").workload

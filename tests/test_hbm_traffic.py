@@ -6,7 +6,8 @@ import os
 
 import pytest
 
-from recflex_amd import hbm_traffic, prebuilt
+from benchaid import hbm_traffic
+from recflex_amd import prebuilt
 
 HEADER = ('"Correlation_Id","Dispatch_Id","Agent_Id","Queue_Id","Process_Id","Thread_Id","Grid_Size",'
           '"Kernel_Id","Kernel_Name","Workgroup_Size","LDS_Block_Size","Scratch_Size","VGPR_Count",'
