@@ -92,6 +92,13 @@ def parse_args() -> argparse.Namespace:
                              "tournament build (0 = rank by tile time only)")
     parser.add_argument("--build_climb_top_k", type=int, default=3,
                         help="build climb: tournament candidates tried per feature")
+    parser.add_argument("--no_cluster_stage", action="store_true", default=False,
+                        help="in-model local stage: stop after the tournament (rank by tile time and "
+                             "its own climb) instead of letting clusters of like features decide on "
+                             "whole-kernel time in production-shaped builds")
+    parser.add_argument("--cluster_top_k", type=int, default=8,
+                        help="cluster stage: candidates a cluster tries")
+    parser.add_argument("--cluster_sweeps", type=int, default=1)
     parser.add_argument("--no_register_census", action="store_true", default=False,
                         help="in-model local stage: admit every candidate to every occupancy's "
                              "tournament, also those that spill registers there")
@@ -163,6 +170,8 @@ def create_tune_config(args: argparse.Namespace) -> TuneConfig:
     else:
         occupancies = list(range(1, max_threads_per_sm // args.block_threads + 1))
     kwargs = {"register_census": not args.no_register_census,
+              "cluster_stage": not args.no_cluster_stage, "cluster_top_k": args.cluster_top_k,
+              "cluster_sweeps": args.cluster_sweeps,
               "build_climb_trials": args.build_climb_trials,
               "build_climb_top_k": args.build_climb_top_k,
               "climb_passes": args.climb_passes, "outliers": {"auto": None, "on": True, "off": False}[args.outliers]}
@@ -210,7 +219,8 @@ def main():
             if args.fixed_thread_binding:
                 fixed_task_blocks, t = tuner.tune_fixed_thread_binding(opt_sched_params=sched_params,
                                                                        choice=args.thread_binding_choice,
-                                                                       tune_config=tune_config)
+                                                                       tune_config=tune_config,
+                                                                       occupancy=occupancy)
                 print(fixed_task_blocks)
                 print(f"Fixed thread binding result: {t/1e6} ms")
 

@@ -214,6 +214,9 @@ int recom_process(const recom_process_args *args);
  * (recom_info.static_workspace == 0) and launches nothing.  Calls no hipMalloc / hipFree or
  * other allocating routine; a small fill kernel ahead of the others puts the array's arrival
  * counters and list header back to zero (no hipMemsetAsync, so the call can be captured).
+ * The first call on a device also resolves the array's address and queries the kernel's
+ * launch state (neither belongs inside a capture): make one eager call per device before
+ * capturing this entry point in a graph.
  * All calls of one library on one device share the one array: calls that may overlap (two
  * streams, two threads) race and must be serialised by the caller.  A library whose
  * recom_get_workspace_bytes() is 0 behaves exactly like recom_process. */

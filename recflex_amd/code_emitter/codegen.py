@@ -199,7 +199,7 @@ class CodeEmitter:
                     timing_branch: bool = False, fixed_task_block_nums: List[int] = None,
                     tile_bytes: int = None, xcd_aware: bool = False,
                     lookup_overhead_bytes: int = None, xcd_segments: int = 8,
-                    outliers: bool = False) -> str:
+                    outliers: bool = False, bind_once: bool = None) -> str:
         num_feats = len(self.feat_schedules)
         if lookup_overhead_bytes is None:
             lookup_overhead_bytes = LOOKUP_OVERHEAD_BYTES
@@ -208,7 +208,8 @@ class CodeEmitter:
         id_map, body_ids = self.dedup()
         flat, cand_begin = self.flat_candidates()
         embed_dim_offsets = self.embed_dim_offsets()
-        bind_once = num_feats > BIND_ONCE_MIN_FEATS
+        if bind_once is None:
+            bind_once = num_feats > BIND_ONCE_MIN_FEATS
         split_regions, workspace_floats = self.split_regions()
         has_split = workspace_floats > 0
         assert not (outliers and (timing or fixed_task_block_nums)), \
@@ -790,11 +791,13 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
              tune: bool = False, timing: bool = False, timing_branch: bool = False,
              fixed_task_block_nums: List[int] = None, tile_bytes: int = None,
              xcd_aware: bool = False, lookup_overhead_bytes: int = None,
-             xcd_segments: int = 8, outliers: bool = False) -> None:
+             xcd_segments: int = 8, outliers: bool = False, bind_once: bool = None) -> None:
         """Write the device source.  ``occupancy`` = workgroups per CU the kernel is built and
         launched for (``__launch_bounds__`` budget, persistent grid size, and a dynamic-LDS pad
         that keeps further workgroups off the CU); ``tune`` is accepted for signature
-        compatibility -- the pad is applied whenever an occupancy is given."""
+        compatibility -- the pad is applied whenever an occupancy is given.  ``bind_once``: bind
+        the model once per launch with a kernel of its own instead of in every workgroup of the
+        fused kernel (None: for models of more than BIND_ONCE_MIN_FEATS features)."""
         code = "// generated by recflex_amd.code_emitter -- do not edit\n"
         code += self.emit_headers()
         code += self.emit_kernel(timing=timing, timing_branch=timing_branch,
@@ -802,7 +805,7 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
                                  fixed_task_block_nums=fixed_task_block_nums,
                                  tile_bytes=tile_bytes, xcd_aware=xcd_aware,
                                  lookup_overhead_bytes=lookup_overhead_bytes,
-                                 xcd_segments=xcd_segments, outliers=outliers)
+                                 xcd_segments=xcd_segments, outliers=outliers, bind_once=bind_once)
         code += self.emit_process_func(timing=timing, occupancy=occupancy)
         code += self.emit_get_concurrent_blocks_func(occupancy=occupancy)
         code += self.emit_process_ops()

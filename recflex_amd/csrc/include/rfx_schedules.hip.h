@@ -21,6 +21,7 @@
 // is a range of bags [bag_begin, bag_end) chosen at run time, and U lookups x UB bags x VPP
 // vectors are kept in flight per lane.
 #pragma once
+#include "rfx_arrival.h"
 #include "rfx_binding.hip.h"
 #include "rfx_crosslane.hip.h"
 #include "rfx_rows.hip.h"
@@ -577,7 +578,7 @@ template <int BT, int DT, int D, int X, int CHUNK> struct BlockBagStorage {
   using R = Row<DT, D>;
   static constexpr int VPL = ceil_div(R::V, X);
   static constexpr int COLS = X * VPL * R::EPV; // >= D
-  int idx[CHUNK];
+  int idx[2][CHUNK];                            // two chunks of indices: one summed, one arriving
   float part[BT / 64][COLS];
   float part_bias[BT / 64];
   int last;                                     // split_bags: this workgroup finishes the bag
@@ -611,13 +612,29 @@ block_sum_range(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict_
 #pragma unroll
     for (int e = 0; e < EPV; ++e) acc[v][e] = 0.f;
 
-  __syncthreads();
-  for (int c0 = beg; c0 < end; c0 += CHUNK) {
-    const int n = min(CHUNK, end - c0);
-    if (c0 != beg) __syncthreads();
+  // The bag's indices pass through LDS in chunks, two buffers taking turns: while the rows of
+  // one chunk are summed, the next chunk's indices are already on their way into registers, and
+  // they are written to the other buffer once this chunk's rows are done.  One barrier per chunk:
+  // a wavefront that writes buffer b for chunk k + 1 has passed the barrier of chunk k, which
+  // every wavefront reaches only after its last read of chunk k - 1 (the earlier tenant of b).
+  constexpr int IPT = CHUNK / BT;               // indices per thread and chunk
+  int arriving[IPT];
+  auto request_chunk = [&](const int c0) {
 #pragma unroll
-    for (int i = 0; i < CHUNK; i += BT)
-      if (i + tid < n) s.idx[i + tid] = indices[c0 + i + tid];
+    for (int i = 0; i < IPT; ++i) {
+      const int p = c0 + i * BT + tid;
+      arriving[i] = indices[p < end ? p : end - 1];      // beyond the bag: a dummy, never used
+    }
+  };
+  if (beg < end) request_chunk(beg);
+  __syncthreads();
+  int cur = 0;
+  for (int c0 = beg; c0 < end; c0 += CHUNK, cur ^= 1) {
+    const int n = min(CHUNK, end - c0);
+    const int *__restrict__ chunk = s.idx[cur];
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) s.idx[cur][i * BT + tid] = arriving[i];
+    if (c0 + CHUNK < end) request_chunk(c0 + CHUNK);
     __syncthreads();
 
     for (int base = 0; base < n; base += U * Y) {
@@ -629,7 +646,7 @@ block_sum_range(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict_
         const int p = base + u * Y + y;
         ok[u] = p < n;
         if (ok[u]) {
-          const char *row = table + static_cast<int64_t>(s.idx[p]) * R::STRIDE;
+          const char *row = table + static_cast<int64_t>(chunk[p]) * R::STRIDE;
 #pragma unroll
           for (int v = 0; v < VPL; ++v) {
             const int c = x + v * X;
@@ -724,6 +741,31 @@ __host__ __device__ constexpr int64_t split_region_floats(int d) {
   return static_cast<int64_t>(kSplitMaxTiles) * (d + 1);
 }
 
+// Memory operations of the arrival protocol on the device.  Partial sums and counters are read
+// and written with device-scope atomic loads and stores: the workgroups of one bag run on
+// different XCDs, whose L2 caches do not see each other's lines otherwise.  A device-scope fence
+// would order them, but it writes back and invalidates the whole L2 of the XCD -- every table row
+// cached there -- for each tile (measured: 6 to 15 times the kernel time of unsplit bags).
+// Device-scope stores are performed at device scope when the memory counter has drained, so
+// waiting for it before the arrival is announced orders the slots before the counter (the
+// release); the finishing workgroup loads the slots only after its arrival has returned (the
+// acquire: every slot load depends on the returned count through the branch on it).
+struct DeviceMem {
+  static __device__ __forceinline__ void store_slot(unsigned int *p, const float v) {
+    __hip_atomic_store(p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  static __device__ __forceinline__ float load_slot(const unsigned int *p) {
+    return __uint_as_float(__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  }
+  static __device__ __forceinline__ void release() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+  static __device__ __forceinline__ int arrive(int *counter) {
+    return __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  static __device__ __forceinline__ void reset(int *counter) {
+    __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+};
+
 // Part `part` of `parts` of bag `bag`: slot p of the bag is slots + p * slot_stride (D values),
 // counter its arrival counter.
 template <int BT, int DT, int D, int X, int U, int CHUNK>
@@ -746,35 +788,21 @@ split_part(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ tab
     return;
   }
 
-  // Partial sums and counters are read and written with device-scope atomic loads and stores:
-  // the workgroups of one bag run on different XCDs, whose L2 caches do not see each other's
-  // lines otherwise.  A device-scope fence would order them, but it writes back and invalidates
-  // the whole L2 of the XCD -- every table row cached there -- for each tile (measured: 6 to 15
-  // times the kernel time of unsplit bags).  Device-scope stores are performed at device scope
-  // when the memory counter has drained, so waiting for it before the arrival is announced
-  // orders the slots before the counter; the finishing workgroup loads the slots only after its
-  // arrival has returned.
+  // The arrival protocol of rfx_arrival.h with the device's memory operations (DeviceMem above).
   for (int j = tid; j < D; j += BT)
-    __hip_atomic_store(slots + static_cast<int64_t>(part) * slot_stride + j,
-                       __float_as_uint(block_column(s, j)), __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    arrival_store<DeviceMem>(slots, part, slot_stride, j, block_column(s, j));
+#ifdef RFX_EXP_NO_ARRIVAL
+  return;
+#endif
+  DeviceMem::release();
   __syncthreads();
-  if (tid == 0) {
-    const int arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s.last = arrived == parts - 1;
-  }
+  if (tid == 0) s.last = arrival_is_last<DeviceMem>(counter, parts);
   __syncthreads();
   if (!s.last) return;              // the same for the whole workgroup
   float *dst = out + static_cast<int64_t>(bag) * esum + col_off;
-  for (int j = tid; j < D; j += BT) {
-    float t = 0.f;
-    for (int p = 0; p < parts; ++p)
-      t += __uint_as_float(__hip_atomic_load(slots + static_cast<int64_t>(p) * slot_stride + j,
-                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-    store_streaming(dst + j, t);
-  }
-  if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (int j = tid; j < D; j += BT)
+    store_streaming(dst + j, arrival_combine<DeviceMem>(slots, parts, slot_stride, j));
+  if (tid == 0) DeviceMem::reset(counter);
 }
 
 template <int BT, int DT, int D, int X, int U, int CHUNK>

@@ -22,6 +22,8 @@ its library is missing.  Names:
                    candidate space of all four templates, with ragged bags (up to ~1500 lookups)
                    and integer-valued tables, so that sums are exact in any order
 ``edge``           dims that force 8- and 4-byte row vectors and unaligned output columns
+``onehots``        the row-copy template at a spread of its candidates for fp32, fp16 and int8
+                   rows, integer-valued tables
 ``longbags``       a dozen samples with bags of thousands of lookups (and some short and empty
                    ones) under the split-bag schedule: several workgroups per bag
 ``c3s_outliers``   c3s with integer-valued tables, emitted with ``outliers=True``: bags beyond a
@@ -187,6 +189,24 @@ def _other_block_size(block_threads: int) -> ModelSpec:
     return ModelSpec(wl, fs, None)
 
 
+def _onehots() -> ModelSpec:
+    """The row-copy template (``OneHotBagSchedule``) for every element type at a spread of its
+    (column lanes, bags per team) candidates.  The workload itself holds exactly one lookup per
+    bag; the tests also feed the library empty bags, bags of many lookups and batches that have
+    as many lookups as bags without having one per bag."""
+    from .schedules import OneHotBagSchedule
+    feats: List[FeatureSpec] = []
+    scheds: FeatSchedules = []
+    for i, (data_type, dim) in enumerate([("float", 64), ("float", 8), ("float", 128), ("half", 32),
+                                          ("half", 128), ("int8", 64), ("int8", 128)]):
+        sched = OneHotBagSchedule(MetaData(dim, data_type), BLOCK_THREADS)
+        cands = sched.GenParamCandidates()
+        for k in sorted(set(int(j) for j in np.linspace(0, len(cands) - 1, min(4, len(cands))))):
+            feats.append(FeatureSpec(700 + 53 * len(feats), dim, data_type, 1.0, True, 0.0, 1.0))
+            scheds.append((sched, cands[k]))
+    return ModelSpec(Workload("onehots", 333, 909, tuple(feats), "integer"), scheds, DEFAULT_OCCUPANCY)
+
+
 def _long_bags() -> ModelSpec:
     """Few, very long bags: every bag of the long features is summed by several workgroups
     (``SplitBagSchedule``); the last two features have short bags and stay unsplit."""
@@ -289,6 +309,7 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c3s_outliers": _c3s_outliers,
     "variants": _variants,
     "edge": _edge,
+    "onehots": _onehots,
     "longbags": _long_bags,
     "c3_skew": lambda: _c3_skew(True),
     "c3_skew_plain": lambda: _c3_skew(False),
@@ -369,7 +390,7 @@ def make_fixture_tuner(model_dir: str, sample_batch_nums: int = 4, codegen_dir: 
 def fixture_tune_config(**overrides):
     from .tuning import TuneConfig
     kwargs = dict(occupancies=TUNE_FIXTURE_OCCUPANCIES, gpu_ids=[0], sm_count=TUNE_FIXTURE_SM_COUNT,
-                  num_processes=4, profiler="events", in_process=True)
+                  num_processes=4, profiler="events", in_process=True, cluster_stage=False)
     kwargs.update(overrides)
     return TuneConfig(**kwargs)
 
@@ -405,7 +426,8 @@ def build_tune_fixture(model_dir: str) -> str:
     mix = fixture_default_mix(tuner)
     tuner.compile_mutation(mix, ABLATION_OCCUPANCY, ABLATION_MUTATED_FEATURE, ablation)
     for choice in ("mean", "max"):
-        tuner.compile_fixed_thread_binding(mix, choice, ablation._replace(remeasure=True))
+        tuner.compile_fixed_thread_binding(mix, choice, ablation._replace(remeasure=True),
+                                           occupancy=ABLATION_OCCUPANCY)
     return tune_fixture_dir()
 
 

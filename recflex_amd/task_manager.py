@@ -50,6 +50,10 @@ class TaskManager:
                 child.start()
                 child.join()
                 code = child.exitcode
+            except Exception as exc:            # e.g. an argument that cannot be pickled: this
+                # task is lost (exit code None), the resource goes on serving the others
+                print(f"TaskManager: could not run {getattr(target, '__name__', target)}: "
+                      f"{type(exc).__name__}: {exc}", flush=True)
             finally:
                 with self._lock:
                     self._busy.remove(resource)

@@ -431,6 +431,44 @@ class KernelTimer:
         return total
 
 
+    def time_options(self, librecom_path: str, members: Sequence[int], num_options: int,
+                     rounds: int = 3, repeats: int = 3, warmup: int = 4, tile_bytes: int = 0,
+                     xcd_segments: int = 0) -> List[List[float]]:
+        """A library that holds ``num_options`` candidates for each feature in ``members`` (and one
+        for every other feature): the whole kernel's time, summed over the batches, with all
+        members on option 0, all on option 1, ...  The options take turns ``rounds`` times, so
+        that a drift of the clocks meets all of them alike; returns the ``rounds`` times (ns) of
+        each option."""
+        import torch
+        from recflex_amd.rec_modules import FeatEmbed
+        layer = FeatEmbed(self.dev, embed_tables=self.tables, librecom=librecom_path)
+        counts = layer.lib.candidate_counts
+        for f in members:
+            if counts[f] != num_options:
+                raise ValueError(f"feature {f} holds {counts[f]} candidates, expected {num_options}")
+        if self.outs is None:
+            self.outs = [layer.forward_indices(d_idx, d_off).clone() for d_idx, d_off in self.batches]
+        bound = [layer.bind_inputs(d_idx, d_off) for d_idx, d_off in self.batches]
+        choices = []
+        for k in range(num_options):
+            c = np.zeros(len(counts), dtype=np.int32)
+            c[list(members)] = k
+            choices.append(torch.from_numpy(c).to(self.dev))
+        times: List[List[float]] = [[] for _ in range(num_options)]
+        for r in range(rounds):
+            for k in range(num_options):
+                total = 0.0
+                for b, out in zip(bound, self.outs):
+                    run = lambda: layer.forward_indices(b, out=out, tile_bytes=tile_bytes,
+                                                        xcd_segments=xcd_segments,
+                                                        schedule_choice=choices[k])
+                    for _ in range(warmup if r == 0 else 1):
+                        run()
+                    total += _timed_launches(run, repeats)
+                times[k].append(total)
+        return times
+
+
 MAX_TILE_FACTOR = 8      # rfx::kMaxTileFactor
 PLENTY_TILES_PER_WORKGROUP = 2                      # rfx::kPlentyTilesPerWorkgroup
 AUTO_TILES_PER_WORKGROUP = 64                       # rfx::kAutoTilesPerWorkgroup
@@ -486,11 +524,14 @@ def tiles_per_feature(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int]
 
 def measure_task_blocks(data_npzs: Sequence[str], lookup_bytes: Sequence[int],
                         bag_bytes: Sequence[int], gran: Sequence[int], tile_bytes: int,
-                        output_path: str) -> None:
-    """One line per batch: comma separated tile counts per feature (CPU only)."""
+                        output_path: str, grid_blocks: int = 0) -> None:
+    """One line per batch: comma separated tile counts per feature (CPU only).  ``grid_blocks``:
+    the workgroups of the grid the counts are for (compute units x occupancy), which the
+    binding's whole-pass rule looks at."""
     per_feat = [load_batches(p) for p in data_npzs]
     lines = []
     for k in range(len(per_feat[0])):
-        tiles = tiles_per_feature([b[k][1] for b in per_feat], lookup_bytes, bag_bytes, gran, tile_bytes)
+        tiles = tiles_per_feature([b[k][1] for b in per_feat], lookup_bytes, bag_bytes, gran, tile_bytes,
+                                  grid_blocks=grid_blocks)
         lines.append(','.join(str(t) for t in tiles))
     _write_atomically(output_path, '\n'.join(lines) + '\n')

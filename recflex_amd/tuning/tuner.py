@@ -34,6 +34,7 @@ import numpy as np
 from recflex_amd.code_emitter import CodeEmitter, ScheduleBase, MetaData
 from recflex_amd.code_emitter.codegen import (BAG_FIXED_BYTES, DEFAULT_TILE_BYTES, INDEX_BYTES,
                                                waves_per_simd)
+from recflex_amd.model_build import DEFAULT_XCD_SEGMENTS
 from recflex_amd.utils import compile_build, os_check
 from recflex_amd.task_manager import TaskManager
 from recflex_amd.parser import (parse_raw_data_batches, parse_table_shapes, parse_table_dtypes,
@@ -87,6 +88,16 @@ class TuneConfig(NamedTuple):
     top_k: int = 8
     # passes of the whole-kernel climb that follows the tile-time tournament (0 = none)
     climb_passes: int = 1
+    # in-model local stage, second half: clusters of like features (same candidate list, same
+    # class of bag length) decide one at a time.  Per cluster a production-shaped build holds the
+    # cluster's ``cluster_top_k`` best-ranked candidates beside the pick of every other feature;
+    # the whole kernel is timed with the cluster on each of them in turn and the cluster adopts
+    # the fastest if it beats its current pick by ``cluster_min_gain``.  ``cluster_sweeps`` passes
+    # over all clusters, heaviest first, ``num_processes`` builds at a time.
+    cluster_stage: bool = True
+    cluster_top_k: int = 8
+    cluster_min_gain: float = 0.004
+    cluster_sweeps: int = 1
     # in-model local stage: compile every distinct candidate body alone for each occupancy and
     # keep out of that occupancy's tournament the ones that spill or come within
     # ``census_margin`` vector registers of the occupancy's budget (they cannot win, and their
@@ -562,7 +573,132 @@ class Tuner:
                 for k, t in zip(admitted[feat_id], times[feat_id]):
                     full[k] = t
                 results[feat_id][occupancy] = full
+        if tune_config.cluster_stage:
+            for occupancy in tune_config.occupancies:
+                picks = self.cluster_stage(occupancy, results, tune_config)
+                for feat_id, k in enumerate(picks):
+                    # an argmin over the scores reproduces the local stage's decision
+                    scores = results[feat_id][occupancy]
+                    finite = [t for t in scores if np.isfinite(t)]
+                    scores[k] = (min(finite) if finite else 1.0) * 0.999
         return results
+
+    # ---- local stage, by clusters of like features ----------------------------------------------
+
+    BAG_LENGTH_CLASSES = (1.5, 4.0, 16.0, 64.0)      # mean lookups per bag: class boundaries
+
+    def feature_clusters(self) -> List[List[int]]:
+        """Features that share a candidate list (element type, dim, templates) and a class of mean
+        bag length, heaviest cluster (by traffic in the sampled batches) first."""
+        groups: Dict[tuple, List[int]] = {}
+        for f in range(self.num_feats):
+            lens = [len(i) / max(1, len(o) - 1) for i, o in self.batches[f]]
+            mean = float(np.mean(lens)) if lens else 0.0
+            cls = sum(mean > b for b in self.BAG_LENGTH_CLASSES)
+            m = self.metas[f]
+            key = (m.data_type, m.embed_dim, len(self.feat_sched_param_candidates[f]),
+                   tuple(type(s).__name__ for s in self.feat_schedules[f]), self.is_one_hot(f), cls)
+            groups.setdefault(key, []).append(f)
+        weight = self.feature_traffic()
+        return sorted(groups.values(), key=lambda g: -float(sum(weight[f] for f in g)))
+
+    def feature_traffic(self) -> np.ndarray:
+        """Bytes each feature moves in the sampled batches (rows + indices + output)."""
+        return np.asarray([sum(len(i) for i, _ in self.batches[f]) * (self.metas[f].row_bytes + INDEX_BYTES)
+                           + self.metas[f].embed_dim * 4 * sum(len(o) - 1 for _, o in self.batches[f])
+                           for f in range(self.num_feats)], dtype=np.float64)
+
+    def cluster_options(self, members: List[int], picks: List[int], occupancy: int,
+                        measured_times: Dict[int, Dict[int, List[float]]], top_k: int) -> List[int]:
+        """The candidates (indices into the members' common candidate list) a cluster tries: the
+        ``top_k`` with the best summed rank scores of the local stage's first half, each
+        member's score taken relative to its own best."""
+        n = len(self.feat_sched_param_candidates[members[0]])
+        total = np.zeros(n)
+        for f in members:
+            sc = np.asarray(measured_times[f][occupancy], dtype=np.float64)
+            finite = sc[np.isfinite(sc)]
+            total += np.where(np.isfinite(sc), sc / (finite.min() if finite.size else 1.0), np.inf)
+        ranked = [int(k) for k in np.argsort(total, kind="stable") if np.isfinite(total[k])]
+        return ranked[:top_k]
+
+    def get_cluster_dir(self, occupancy: int, sweep: int, cluster: int) -> str:
+        return f"{self.basic.codegen_dir}/clusters/o{occupancy}/s{sweep}_c{cluster}"
+
+    def cluster_stage(self, occupancy: int, measured_times: Dict[int, Dict[int, List[float]]],
+                      tune_config: TuneConfig) -> List[int]:
+        """Second half of the in-model local stage (see ``TuneConfig.cluster_stage``).  Starts
+        from the default-heuristic mix (each pick moved to the nearest candidate the register
+        census admits at this occupancy); returns the index of every feature's pick in its
+        candidate list.  ``clusters/o{occ}/result.json`` keeps what was measured."""
+        result_log = f"{self.basic.codegen_dir}/clusters/o{occupancy}/result.json"
+        if os.path.exists(result_log) and not tune_config.remeasure:
+            with open(result_log) as f:
+                return json.load(f)["picks"]
+        admitted = self.admitted_candidates(occupancy)
+        picks = [admitted[f][self._nearest_admitted(f, k, admitted[f])]
+                 for f, k in enumerate(self.default_choices()[0])]
+        start = list(picks)
+        clusters = self.feature_clusters()
+        timer = KernelTimer(self.table_shapes, self.data_types, self.data_npzs,
+                            gpu_id=tune_config.gpu_ids[0])
+        width = max(1, tune_config.num_processes)
+        log = []
+        for sweep in range(tune_config.cluster_sweeps):
+            changed = False
+            for lo in range(0, len(clusters), width):
+                group = list(enumerate(clusters))[lo:lo + width]
+                builds = []
+                jobs = []
+                for ci, members in group:
+                    options = self.cluster_options(members, picks, occupancy, measured_times,
+                                                   tune_config.cluster_top_k)
+                    if not options:
+                        continue
+                    # option 0: every member keeps its pick; option j: all members run options[j-1]
+                    cands = [[self.feat_sched_param_candidates[f][picks[f]]] for f in range(self.num_feats)]
+                    for f in members:
+                        cands[f] += [self.feat_sched_param_candidates[f][k] for k in options]
+                    out = self.get_cluster_dir(occupancy, sweep, ci)
+                    if not self._kept(out, tune_config) or not os.path.exists(f"{out}/options.json"):
+                        os.makedirs(f"{out}/build", exist_ok=True)
+                        emitter = CodeEmitter(None, feat_candidates=cands)
+                        emitter.emit(f"{out}/process.hip", occupancy=occupancy, inline=tune_config.inline,
+                                     tune=True, tile_bytes=tune_config.tile_bytes)
+                        emitter.emit_cmake_list(f"{out}/CMakeLists.txt", code_fname="process.hip",
+                                                host_fname=None, subdirs=self.basic.subdirs,
+                                                includes=self.basic.includes, links=self.basic.links,
+                                                debug=tune_config.debug)
+                        with open(f"{out}/options.json", "w") as f:
+                            json.dump({"members": members, "options": options,
+                                       "picks": [picks[f] for f in members]}, f)
+                        jobs.append((out, f"{out}/build"))
+                    builds.append((ci, members, options, out))
+                self._schedule_builds(jobs, tune_config)
+                for ci, members, options, out in builds:
+                    times = timer.time_options(f"{out}/build/librecom.so", members, len(options) + 1,
+                                               xcd_segments=DEFAULT_XCD_SEGMENTS)
+                    med = [float(np.median(t)) for t in times]
+                    best = int(np.argmin(med))
+                    gain = 1.0 - med[best] / med[0]
+                    adopt = best > 0 and gain >= tune_config.cluster_min_gain
+                    log.append({"sweep": sweep, "cluster": ci, "members": members,
+                                "options": options, "kept_picks": [picks[f] for f in members],
+                                "kernel_ns": med, "adopted": options[best - 1] if adopt else None})
+                    print(f"[clusters {occupancy}] sweep {sweep} cluster {ci} ({len(members)} features, "
+                          f"dim {self.metas[members[0]].embed_dim}): kept {med[0]:.0f} ns, best option "
+                          f"{med[best]:.0f} ns ({100 * gain:.2f} %)" + (" -> adopted" if adopt else ""),
+                          flush=True)
+                    if adopt:
+                        for f in members:
+                            picks[f] = options[best - 1]
+                        changed = True
+            if not changed:
+                break
+        os.makedirs(os.path.dirname(result_log), exist_ok=True)
+        with open(result_log, "w") as f:
+            json.dump({"picks": picks, "start": start, "clusters": log}, f)
+        return picks
 
     def _nearest_admitted(self, feat_id: int, pick: int, admitted: List[int]) -> int:
         """Position, in the admitted list, of candidate ``pick`` of the feature -- or of the
@@ -1018,7 +1154,8 @@ class Tuner:
         return opt_sched_params, self._read_kernel_time(output_dir, tune_config)
 
     def compile_fixed_thread_binding(self, opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]],
-                                     choice: str, tune_config: TuneConfig) -> List[int]:
+                                     choice: str, tune_config: TuneConfig,
+                                     occupancy: int = None) -> List[int]:
         """Write ``fixed_thread_binding_{choice}/task_blocks.txt`` (the tiles per feature the
         run-time binding would choose for each sampled batch, computed on the CPU), freeze their
         mean / max into a kernel and build it (no GPU needed).  Returns the frozen counts."""
@@ -1032,7 +1169,8 @@ class Tuner:
                                 [m.row_bytes + INDEX_BYTES for m in metas],
                                 [m.embed_dim * 4 + BAG_FIXED_BYTES for m in metas],
                                 [s.TileGranularity(p) for s, p in opt_sched_params],
-                                tune_config.tile_bytes, fixed_blocks_path)
+                                tune_config.tile_bytes, fixed_blocks_path,
+                                grid_blocks=tune_config.sm_count * (occupancy or self.natural_occupancy_guess()))
 
         task_block_batches: List[List[int]] = []
         with open(fixed_blocks_path) as f:
@@ -1046,16 +1184,26 @@ class Tuner:
             fixed_task_blocks: List[int] = np.mean(task_block_batches, axis=0, dtype=np.int32).tolist()
         fixed_task_blocks = [max(1, int(b)) for b in fixed_task_blocks]
 
-        if self._build_full(output_dir, opt_sched_params, None, tune_config,
+        if self._build_full(output_dir, opt_sched_params, occupancy, tune_config,
                             fixed_task_block_nums=fixed_task_blocks):
             self._schedule_builds([(output_dir, f"{output_dir}/build")], tune_config)
         return fixed_task_blocks
 
+    def natural_occupancy_guess(self) -> int:
+        """Workgroups per CU of a library emitted without an occupancy (the frozen-binding
+        ablation is): the grid the run-time binding of such a library sees is compute units x
+        this.  The fused kernels here use 64 to 128 vector registers, which is 4 workgroups of
+        256 threads per CU; other workgroup sizes scale."""
+        return max(1, 4 * 256 // max(64, self.basic.block_threads))
+
     def tune_fixed_thread_binding(self, opt_sched_params: List[Tuple[ScheduleBase, NamedTuple]], choice: str,
-                                  tune_config: TuneConfig) -> Tuple[List[int], float]:
+                                  tune_config: TuneConfig, occupancy: int = None) -> Tuple[List[int], float]:
         """Ablation: the number of tiles per feature is frozen to the mean / max over the sampled
-        batches of what the run-time binding chose, and baked into the kernel."""
-        fixed_task_blocks = self.compile_fixed_thread_binding(opt_sched_params, choice, tune_config)
+        batches of what the run-time binding chose, and baked into the kernel.  ``occupancy``:
+        the workgroups per CU of the run-time-bound library it is compared with (its grid enters
+        the binding's rules)."""
+        fixed_task_blocks = self.compile_fixed_thread_binding(opt_sched_params, choice, tune_config,
+                                                              occupancy)
         output_dir = f"{self.basic.codegen_dir}/fixed_thread_binding_{choice}"
         manager = self._measure_manager(tune_config)
         self._kernel_time(output_dir, tune_config, manager)

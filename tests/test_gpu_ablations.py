@@ -74,7 +74,7 @@ def test_fixed_thread_binding(choice):
     cfg = prebuilt.fixture_tune_config(tile_bytes=prebuilt.ABLATION_TILE_BYTES, remeasure=False)
     mix = prebuilt.fixture_default_mix(tuner)
     print(f"[case] fixed thread binding, choice={choice}", flush=True)
-    fixed, t_ns = tuner.tune_fixed_thread_binding(mix, choice, cfg)
+    fixed, t_ns = tuner.tune_fixed_thread_binding(mix, choice, cfg, occupancy=prebuilt.ABLATION_OCCUPANCY)
     assert len(fixed) == tuner.num_feats and all(b >= 1 for b in fixed) and t_ns > 0
     # the frozen counts are the mean / max of the per-batch lines (which the CPU wrote)
     lines = [list(map(int, ln.split(","))) for ln in

@@ -68,7 +68,7 @@ def test_binding_is_result_invariant(tile_bytes, grid, xcd):
     _assert_parity(*_run_model("c3s", tile_bytes=tile_bytes, grid_blocks=grid, xcd_segments=xcd))
 
 
-@pytest.mark.parametrize("name", ["variants", "edge", "wide", "wider", "longbags"])
+@pytest.mark.parametrize("name", ["variants", "edge", "onehots", "wide", "wider", "longbags"])
 def test_integer_tables_are_bit_exact(name):
     """Integer-valued tables make every fp32 sum exact, so each schedule variant (any lane
     split, any reduction tree) must reproduce the oracle's bits."""
@@ -216,6 +216,61 @@ def test_onehot_is_bit_exact():
     """Bags of exactly one lookup are a row copy: identical bits (C2 shape, shrunk)."""
     wl, got, want = _run_model("c2s")
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("case", ["one_each", "as_many_lookups_as_bags", "zero_or_one", "ragged",
+                                  "one_long_among_ones", "all_empty"])
+@pytest.mark.parametrize("batch", [1, 77, 1024])
+def test_row_copy_template_on_any_input(case, batch):
+    """``rfx::onehot_bags`` (``OneHotBagSchedule``, 28 candidates over fp32 / fp16 / int8 rows) on
+    inputs it is and is not meant for: exactly one lookup per bag (the hint holds: an index is
+    fetched together with its bag's offsets); as many lookups as bags but lengths 2, 0, 1, ...
+    (the hint is set and wrong); bags of zero or one lookup (no hint); empty bags beside bags of
+    2 to 100 lookups (the pass goes to the team routine with a per-wavefront stage slice); one
+    bag of 500 lookups among bags of one (handed on to a whole wavefront); no lookup at all.
+    Integer-valued tables: bit for bit, for every element type (row copy, scale and bias,
+    staged output)."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_tables
+
+    wl = prebuilt.model_spec("onehots").workload
+    assert wl.table_values == "integer" and wl.num_features <= 512      # the hint is live
+    dev = torch.device("cuda", 0)
+    print(f"[case] onehots, {case}, B={batch}", flush=True)
+    rng = np.random.default_rng(batch * 31 + len(case))
+    tables = gen_tables(wl, dev)
+    indices, offsets = [], []
+    for f, spec in enumerate(wl.features):
+        if case == "one_each":
+            lens = np.ones(batch, dtype=np.int64)
+        elif case == "as_many_lookups_as_bags":
+            lens = np.ones(batch, dtype=np.int64)
+            for b in range(f % 3, batch - 1, 3):           # 2, 0 in place of 1, 1
+                lens[b], lens[b + 1] = 2, 0
+        elif case == "zero_or_one":
+            lens = (rng.random(batch) < 0.7).astype(np.int64)
+        elif case == "ragged":
+            lens = rng.integers(2, 101, batch) * (rng.random(batch) < 0.5)
+        elif case == "one_long_among_ones":
+            lens = np.ones(batch, dtype=np.int64)
+            lens[rng.integers(0, batch)] = 500
+        else:
+            lens = np.zeros(batch, dtype=np.int64)
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        if case == "as_many_lookups_as_bags":
+            assert off[-1] == batch
+        indices.append(rng.integers(0, spec.rows, int(off[-1])).astype(np.int32))
+        offsets.append(off)
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib("onehots"))
+    d_idx = [torch.from_numpy(i).to(dev) for i in indices]
+    d_off = [torch.from_numpy(o).to(dev) for o in offsets]
+    got = layer.forward_indices(d_idx, d_off).cpu().numpy()
+    want = oracle_output(wl._replace(batch=batch), [t.cpu().numpy() for t in tables], indices, offsets)
+    assert got.shape == want.shape == (batch, wl.embed_dim_sum)
+    bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+    assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
 
 
 def test_gather_probe_runs():

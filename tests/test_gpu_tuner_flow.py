@@ -122,6 +122,50 @@ def test_tournament_then_global_stage():
     _check_text_model(model, tuner, raw_batches)
 
 
+def test_cluster_stage_decides_the_local_stage():
+    """The local stage's second half: clusters of like features try their best-ranked candidates
+    in production-shaped builds (compiled here: one small kernel per cluster) and decide on
+    whole-kernel time; the scores ``tune`` returns elect exactly that mix, and the library the
+    global stage builds from it computes the right thing."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.parser import parse_raw_data_batches
+    from recflex_amd.rec_modules import FeatProcessEmbed
+    from recflex_amd.host import RecomHost
+    if shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"):
+        pytest.skip("the cluster stage builds one kernel per cluster and needs hipcc")
+    d, tuner = _fixture()
+    shutil.rmtree(os.path.join(d, "clusters"), ignore_errors=True)
+    cfg = prebuilt.fixture_tune_config(interference="model", occupancies=[4], remeasure=True, rounds=1,
+                                       refine_passes=1, climb_passes=0, cluster_stage=True,
+                                       cluster_top_k=3, cluster_min_gain=0.0, include_default=False)
+    print("[case] tournament + cluster stage at 4 workgroups per CU", flush=True)
+    res = tuner.tune(cfg)
+    doc = json.load(open(os.path.join(d, "clusters", "o4", "result.json")))
+    clusters = tuner.feature_clusters()
+    assert sorted(f for c in clusters for f in c) == list(range(6))
+    assert len(doc["clusters"]) == len(clusters) and len(doc["picks"]) == 6
+    admitted = tuner.admitted_candidates(4)
+    for entry in doc["clusters"]:
+        assert len(entry["kernel_ns"]) == len(entry["options"]) + 1 and min(entry["kernel_ns"]) > 0
+        assert all(k in admitted[f] for f in entry["members"] for k in entry["options"])
+        if entry["adopted"] is not None:           # with no minimum gain: the fastest option
+            assert entry["adopted"] == entry["options"][int(np.argmin(entry["kernel_ns"])) - 1]
+            assert all(doc["picks"][f] == entry["adopted"] for f in entry["members"])
+    for f in range(6):
+        assert int(np.argmin(res[f][4])) == doc["picks"][f]
+    print("[case] global stage on the elected mix (builds 1 small kernel)", flush=True)
+    occ, sched = tuner.solve(res, cfg)
+    assert occ == 4
+    for f in range(6):
+        assert sched[f] is tuner.feat_sched_param_candidates[f][doc["picks"][f]]
+    raw_batches = parse_raw_data_batches(tuner.basic.batch_sizes_fname, tuner.basic.data_fnames, 2,
+                                         seed=2, feat_major=False)
+    model = FeatProcessEmbed(RecomHost(), torch.device("cuda", 0), table_shapes=tuner.table_shapes,
+                             librecom_path=os.path.join(d, "optimal", "build", "librecom.so"))
+    _check_text_model(model, tuner, raw_batches)
+
+
 def test_compressed_model_flow():
     """``examples/run_model.sh``: the model is compressed to one representative per cluster of
     like features (``compress.py``), the representatives' candidates are measured (``tune.py

@@ -188,6 +188,29 @@ def test_task_manager_returns_resources_and_survives_failures(tmp_path):
     assert sorted(tm.exit_codes) == [0, 0, 0, 0, 0, 1]
 
 
+def test_task_manager_outlives_a_task_it_cannot_start(tmp_path):
+    """An argument that cannot be pickled (spawn) loses that one task: the single resource keeps
+    serving, join() returns, and a second round of tasks runs too."""
+    import threading
+    from recflex_amd.task_manager import TaskManager
+    if mp.get_start_method(allow_none=True) != "spawn":
+        mp.set_start_method("spawn", force=True)
+    log = str(tmp_path / "log.txt")
+    tm = TaskManager(["only"])
+    tm.add_task(_sleep_and_record, (log,), ident_key="ident")
+    tm.add_task(_sleep_and_record, (threading.Lock(),), ident_key="ident")      # not picklable
+    tm.add_task(_sleep_and_record, (log,), ident_key="ident")
+    done = threading.Thread(target=tm.join, daemon=True)
+    done.start()
+    done.join(60)
+    assert not done.is_alive(), "join() hangs after a task that could not be started"
+    assert open(log).read().split() == ["only", "only"]
+    assert sorted(tm.exit_codes, key=str) == [0, 0, None]
+    tm.add_task(_sleep_and_record, (log,), ident_key="ident")                   # the next round
+    tm.join()
+    assert len(open(log).read().split()) == 3 and tm.resource_queue.qsize() == 1
+
+
 def test_register_census_filters_the_tournament(tmp_path, monkeypatch):
     """Candidates that spill, or come within the margin of the occupancy's register budget, stay
     out of that occupancy's tournament; results are mapped back to the full candidate lists."""
@@ -393,6 +416,83 @@ def test_whole_passes_when_tiles_are_plentiful():
     assert tiles_per_feature(*args, grid_blocks=1280)[0] == 512  # 512 * 100 >= 2 * 1280
     few = ([off[:33]] * 4, [516] * 4, [516] * 4, [4] * 4, 65536)
     assert tiles_per_feature(*few, grid_blocks=1280)[0] == 32    # 8 * 4 < 2 * 1280: spread out
+
+
+def test_cluster_stage_adopts_by_whole_kernel_time(tmp_path, monkeypatch):
+    """Local stage by clusters: like features form one cluster, a cluster tries its best-ranked
+    candidates and adopts the one that makes the whole kernel faster by the minimum gain -- and
+    keeps its picks otherwise; an argmin over the returned scores reproduces the decision.
+    (No compiler and no GPU: builds and kernel times are stand-ins.)"""
+    import recflex_amd.tuning.tuner as tuner_mod
+    rng = np.random.default_rng(3)
+    data = []
+    for f in range(5):
+        mean = [1, 1, 30, 30, 300][f]
+        bl = []
+        for _ in range(2):
+            lens = np.full(16, mean) if mean == 1 else rng.poisson(mean, 16)
+            off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            bl.append((rng.integers(0, 100, off[-1]).astype(np.int32), off))
+        data.append(bl)
+    cfg = BasicConfig("", [], "", "", str(tmp_path / "out"), block_threads=256, sample_batch_nums=2)
+    t = Tuner(cfg, SCHEDULE_MAPPING, batches=data, table_shapes=[(100, 16)] * 5, data_types=["float"] * 5,
+              schedule_types=[[WarpPerSampleSchedule]] * 5)
+    clusters = t.feature_clusters()
+    assert sorted(map(sorted, clusters)) == [[0, 1], [2, 3], [4]]
+    assert clusters[0] == [4]                                  # the heaviest cluster first
+    n = len(t.feat_sched_param_candidates[0])
+    tc = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=2, in_process=True,
+                    register_census=False, cluster_top_k=3, cluster_min_gain=0.01)
+    # rank scores of the first half: candidate 5 best for every feature, then 2, then 7
+    scores = np.full(n, 10.0)
+    scores[[5, 2, 7]] = [1.0, 2.0, 3.0]
+    measured = {f: {4: scores.tolist()} for f in range(5)}
+    assert t.cluster_options([2, 3], [0] * 5, 4, measured, 3) == [5, 2, 7]
+
+    monkeypatch.setattr(Tuner, "_schedule_builds", lambda self, jobs, cfg_: None)
+    monkeypatch.setattr(Tuner, "_kept", lambda self, out, cfg_: False)
+    asked = []
+
+    class FakeTimer:
+        def __init__(self, *a, **k):
+            pass
+
+        def time_options(self, lib, members, num_options, **kw):
+            asked.append((tuple(members), num_options))
+            base = [[100.0] * 3 for _ in range(num_options)]
+            if tuple(members) == (4,):
+                base[2] = [90.0, 91.0, 89.0]                   # option 2 (candidate 2): 10 % faster
+            if tuple(members) == (2, 3):
+                base[1] = [99.8, 99.9, 99.7]                   # 0.2 %: below the minimum gain
+            return base
+
+    monkeypatch.setattr(tuner_mod, "KernelTimer", FakeTimer)
+    start = [t._nearest_admitted(f, k, list(range(n))) for f, k in enumerate(t.default_choices()[0])]
+    picks = t.cluster_stage(4, measured, tc)
+    assert asked == [((4,), 4), ((2, 3), 4), ((0, 1), 4)]
+    assert picks[4] == 2 and picks[:4] == start[:4]
+    doc = json.load(open(tmp_path / "out" / "clusters" / "o4" / "result.json"))
+    assert doc["picks"] == picks and [c["adopted"] for c in doc["clusters"]] == [2, None, None]
+    # a second call reads the result file
+    monkeypatch.setattr(tuner_mod, "KernelTimer", None)
+    assert t.cluster_stage(4, measured, tc) == picks
+
+
+def test_task_blocks_of_the_frozen_binding_see_the_grid(tmp_path):
+    """measure_task_blocks hands the grid (compute units x occupancy) to the host restatement of
+    the binding, so the frozen counts are the ones the run-time binding chooses on that grid."""
+    from recflex_amd.tuning.measure import measure_task_blocks, save_batches
+    off = np.arange(0, 2049 * 320, 320, dtype=np.int32)
+    idx = np.zeros(int(off[-1]), dtype=np.int32)
+    paths = []
+    for f in range(100):
+        paths.append(str(tmp_path / f"f{f}.npz"))
+        save_batches(paths[-1], [(idx, off)])
+    args = (paths, [516] * 100, [516] * 100, [4] * 100, 65536)
+    measure_task_blocks(*args, str(tmp_path / "unknown.txt"))
+    measure_task_blocks(*args, str(tmp_path / "grid.txt"), grid_blocks=256 * 5)
+    assert open(tmp_path / "unknown.txt").read().split(",")[0] == "2048"
+    assert open(tmp_path / "grid.txt").read().split(",")[0] == "512"
 
 
 def test_an_existing_library_is_kept_only_if_it_is_the_build_of_todays_sources(tmp_path, monkeypatch):
