@@ -48,9 +48,16 @@ INDEX_BYTES = 4
 # trip), expressed here as extra bytes so that tiles of narrow-row features do not run longer
 # than tiles of wide-row features.
 LOOKUP_OVERHEAD_BYTES = 0
-# models of more features than this are bound once per launch by a small kernel instead of by
-# every workgroup of the fused kernel (rfx::bind_once)
-BIND_ONCE_MIN_FEATS = 2048
+# Models of more features than this are bound once per launch by a small kernel instead of by
+# every workgroup of the fused kernel (rfx::bind_once), unless the emitter is told otherwise.
+# Up to rfx::kBindKeepAddrs (512) features a workgroup's own binding also leaves every feature's
+# addresses in LDS for its tiles; beyond, a tile reads them from memory either way and the
+# per-workgroup binding is only repeated work -- a thousand workgroups asking for the same two
+# cache lines per feature.  Measured on models of 256-bag batches of small features at four
+# workgroups per CU (per workgroup -> once per launch): 600 features 75.3 -> 72.0 us, 800
+# features 75.4 -> 70.6, 1 000 features 80.8 -> 75.1 (and 29.9 -> 28.8 at 300).  The
+# per-workgroup binding cannot hold more than 2 048 features in LDS beside four workgroups per CU.
+BIND_ONCE_MIN_FEATS = 512
 # a bag becomes tiles of its own (libraries emitted with outliers=True) from this much traffic
 OUTLIER_MIN_BYTES = 128 * 1024
 

@@ -41,12 +41,24 @@ template <class Mem> RFX_ARRIVAL_FN bool arrival_is_last(int *counter, const int
   return Mem::arrive(counter) == parts - 1;
 }
 
-// Column j of the bag: the parts' values added in part order, whoever arrived last.
+// Column j of the bag: the parts' values added in part order, whoever arrived last.  The slot
+// loads are issued eight at a time and only then added: one after the other, each a round trip to
+// the device's coherence point, they made the last arrival of every bag the tail of the kernel.
 template <class Mem>
 RFX_ARRIVAL_FN float arrival_combine(const unsigned int *slots, const int parts,
                                      const int slot_stride, const int j) {
+  constexpr int kBurst = 8;
   float t = 0.f;
-  for (int p = 0; p < parts; ++p) t += Mem::load_slot(slots + static_cast<long long>(p) * slot_stride + j);
+  int p = 0;
+  for (; p + kBurst <= parts; p += kBurst) {
+    float v[kBurst];
+#pragma unroll
+    for (int k = 0; k < kBurst; ++k)
+      v[k] = Mem::load_slot(slots + static_cast<long long>(p + k) * slot_stride + j);
+#pragma unroll
+    for (int k = 0; k < kBurst; ++k) t += v[k];
+  }
+  for (; p < parts; ++p) t += Mem::load_slot(slots + static_cast<long long>(p) * slot_stride + j);
   return t;
 }
 

@@ -84,6 +84,12 @@ struct IoView {
 // 161 us at four workgroups per CU, with 256 KiB parts 142 / 103 / 122 us; at eight workgroups
 // per CU, which these light kernels allow, 138 / 76 / 83 us and 107 / 83 / 96 us).
 constexpr int kSplitMinUnit = 256 * 1024;
+// ... unless the batch is so small that parts of that size leave the workgroups with one or two
+// tiles each: then the part size is chosen so that the tiles come out as a whole number per
+// workgroup, down to kSplitFloorUnit (16 x 20 000 lookups on 2 048 workgroups: 2 880 parts of
+// 256 KiB are 1.4 tiles per workgroup, i.e. two rounds with the second a third full, 94 us;
+// 3 872 parts of 199 KiB are 1.9, 88 us).
+constexpr int kSplitFloorUnit = 128 * 1024;
 constexpr int kSplitGran = -1;
 constexpr int kBindMaxParts = 64;
 constexpr int kBindMaxSplitTiles = 2048;
@@ -231,7 +237,8 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     const int f = min(tid + k * BT, F - 1);
     io.addrs(f, idx_at[k], offs_at[k]);
     table_at[k] = 0;
-    if constexpr (BindingStorage<F>::kKeepAddrs) table_at[k] = table_ptrs[f];
+    // (the once-per-launch binding kernel has no use for the tables' addresses and passes none)
+    if constexpr (BindingStorage<F>::kKeepAddrs) table_at[k] = table_ptrs ? table_ptrs[f] : 0;
     cand[k] = f;
     if constexpr (!ONE_CAND) {
       const int first = cand_begin[f];
@@ -286,9 +293,19 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     const long long total_bytes = static_cast<long long>(total);
     if (automatic) tile_size = auto_tile_size(total_bytes, grid_blocks);
     if (SPLIT) {
-      split_unit = total_bytes / (4ll * (grid_blocks > 0 ? grid_blocks : 1));
+      const long long grid = grid_blocks > 0 ? grid_blocks : 1;
+      split_unit = total_bytes / (4ll * grid);
       if (split_unit < tile_size) split_unit = tile_size;
-      if (split_unit < kSplitMinUnit) split_unit = kSplitMinUnit;
+      if (split_unit < kSplitMinUnit) {
+        // whole tiles per workgroup at about the minimum part size, and 6 % of slack for the
+        // rounding up of every feature's parts per bag
+        const long long per_workgroup = (total_bytes + grid * kSplitMinUnit - 1) / (grid * kSplitMinUnit);
+        split_unit = total_bytes / (grid * (per_workgroup > 0 ? per_workgroup : 1));
+        split_unit += split_unit >> 4;
+        if (split_unit > kSplitMinUnit) split_unit = kSplitMinUnit;
+        if (split_unit < kSplitFloorUnit) split_unit = kSplitFloorUnit;
+        if (split_unit < tile_size) split_unit = tile_size;
+      }
     }
   }
 
@@ -308,7 +325,9 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     int tiles = want < 1 ? 1 : (want > B ? B : static_cast<int>(want));
     int bpt = 0;
     int64_t parts = 1;
-    if (SPLIT && may_split && B > 0 && split_unit > 0 && bag_cost > 2 * split_unit) {
+    // a bag is split from 1.25 units on (128 x 2 500 lookups: 102.8 us with bags of 1.7 units left
+    // whole beside split ones, 89.3 us with those in two parts)
+    if (SPLIT && may_split && B > 0 && split_unit > 0 && 4 * bag_cost > 5 * split_unit) {
       parts = approx_ceil_div(bag_cost, split_unit);
       if (parts > kBindMaxParts) parts = kBindMaxParts;
       if (parts * B > kBindMaxSplitTiles) parts = kBindMaxSplitTiles / B;

@@ -791,9 +791,6 @@ split_part(BlockBagStorage<BT, DT, D, X, CHUNK> &s, const char *__restrict__ tab
   // The arrival protocol of rfx_arrival.h with the device's memory operations (DeviceMem above).
   for (int j = tid; j < D; j += BT)
     arrival_store<DeviceMem>(slots, part, slot_stride, j, block_column(s, j));
-#ifdef RFX_EXP_NO_ARRIVAL
-  return;
-#endif
   DeviceMem::release();
   __syncthreads();
   if (tid == 0) s.last = arrival_is_last<DeviceMem>(counter, parts);

@@ -26,6 +26,8 @@ its library is missing.  Names:
                    rows, integer-valued tables
 ``longbags``       a dozen samples with bags of thousands of lookups (and some short and empty
                    ones) under the split-bag schedule: several workgroups per bag
+``c3s_bind_once``  c3s bound once per launch by the binding kernel (``bind_once=True``), although
+                   small enough for the per-workgroup binding
 ``c3s_outliers``   c3s with integer-valued tables, emitted with ``outliers=True``: bags beyond a
                    schedule's threshold are found ahead of the kernel and run as tiles of their
                    own; every tenth feature under the split-bag schedule
@@ -39,7 +41,8 @@ its library is missing.  Names:
 ``refa``, ``reff4`` models shaped like the reference's example models A and a quarter of F (1 000 and
                    2 500 small features, batch 256; ``workloads.REF_SHAPED``), default schedules;
                    ``refa_tuned``: with ``tuned/refa_schedule.json`` if that file exists
-``wide``           1 500 small features (several binding rounds per thread)
+``wide``           1 500 small features, bound by every workgroup (``bind_once=False``: several
+                   binding rounds per thread)
 ``wider``          2 500 small features (bound once per launch by the binding kernel)
 """
 
@@ -280,7 +283,9 @@ def _wide(num_features: int = 1500, name: str = "wide") -> ModelSpec:
         feats.append(FeatureSpec(int(rng.integers(64, 512)), dim, "float", mean, mean == 1.0,
                                  0.0 if mean == 1.0 else 0.3, 1.05))
     wl = Workload(name, 40, num_features, tuple(feats), "integer")
-    return _default(wl)
+    # wide: bound by every workgroup (several rounds of the binding loop per thread); wider: by
+    # the binding kernel
+    return _default(wl, bind_once=num_features > 2048)
 
 
 _SPECS: Dict[str, Callable[[], ModelSpec]] = {
@@ -306,6 +311,9 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c3s": lambda: _default(make_workload("C3", batch=192, max_rows=60_000)),
     "c4s": lambda: _default(make_workload("C4", batch=128, num_features=48, max_rows=30_000)),
     "c5s": lambda: _default(make_workload("C5", batch=256, num_features=24, max_rows=50_000)),
+    # a model of fewer features than the binding keeps addresses for in LDS, bound once per launch
+    # by the binding kernel all the same (an emit option)
+    "c3s_bind_once": lambda: _default(make_workload("C3", batch=192, max_rows=60_000), bind_once=True),
     "c3s_outliers": _c3s_outliers,
     "variants": _variants,
     "edge": _edge,

@@ -103,7 +103,8 @@ def test_resume_uses_existing_results(tmp_path):
 def test_tournament_results_are_read_back(tmp_path):
     """Default local stage: one result.json per occupancy under tournament/o{occ}."""
     t = _tiny_tuner(tmp_path)
-    cfg = TuneConfig(occupancies=[2, 4], gpu_ids=[0], sm_count=4, num_processes=1, in_process=True)
+    cfg = TuneConfig(occupancies=[2, 4], gpu_ids=[0], sm_count=4, num_processes=1, in_process=True,
+                     cluster_stage=False)      # the tournament alone: the cluster stage measures on a GPU
     counts = [len(c) for c in t.feat_sched_param_candidates]
     for occ in (2, 4):
         out, build_dir = t.get_tournament_dir(occ)
@@ -245,7 +246,7 @@ def test_register_census_filters_the_tournament(tmp_path, monkeypatch):
         json.dump(admitted, fh)
     with open(f"{out}/result.json", "w") as fh:
         json.dump({"times": [[float(j + 1) for j in range(len(k))] for k in admitted]}, fh)
-    res = t.tune(cfg)
+    res = t.tune(cfg._replace(cluster_stage=False))      # the tournament's scores as they are
     for feat, keep in enumerate(admitted):
         full = res[feat][4]
         assert len(full) == len(t.feat_sched_param_candidates[feat])
