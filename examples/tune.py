@@ -96,6 +96,13 @@ def parse_args() -> argparse.Namespace:
                         help="in-model local stage: stop after the tournament (rank by tile time and "
                              "its own climb) instead of letting clusters of like features decide on "
                              "whole-kernel time in production-shaped builds")
+    parser.add_argument("--incumbent", type=str,
+                        help="schedule.json of an earlier tuning run of this model: one more contender of "
+                             "the global stage (and the start of the build climb if it wins)")
+    parser.add_argument("--validate_clusters", action="store_true", default=False,
+                        help="after tuning: build, for every cluster, the production kernel with and "
+                             "without the cluster's fastest option and set the change beside the one "
+                             "the cluster stage measured (clusters/o<occ>/validation.json)")
     parser.add_argument("--cluster_top_k", type=int, default=8,
                         help="cluster stage: candidates a cluster tries")
     parser.add_argument("--cluster_sweeps", type=int, default=1)
@@ -171,7 +178,7 @@ def create_tune_config(args: argparse.Namespace) -> TuneConfig:
         occupancies = list(range(1, max_threads_per_sm // args.block_threads + 1))
     kwargs = {"register_census": not args.no_register_census,
               "cluster_stage": not args.no_cluster_stage, "cluster_top_k": args.cluster_top_k,
-              "cluster_sweeps": args.cluster_sweeps,
+              "cluster_sweeps": args.cluster_sweeps, "incumbent": args.incumbent,
               "build_climb_trials": args.build_climb_trials,
               "build_climb_top_k": args.build_climb_top_k,
               "climb_passes": args.climb_passes, "outliers": {"auto": None, "on": True, "off": False}[args.outliers]}
@@ -215,6 +222,8 @@ def main():
         if not args.local_only:
             occupancy, sched_params = tuner.solve(tune_results, tune_config)
             print(occupancy, sched_params)
+            if args.validate_clusters and tune_config.interference == "model" and tune_config.cluster_stage:
+                tuner.cluster_validation(occupancy, tune_config)
 
             if args.fixed_thread_binding:
                 fixed_task_blocks, t = tuner.tune_fixed_thread_binding(opt_sched_params=sched_params,

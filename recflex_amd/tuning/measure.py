@@ -433,39 +433,61 @@ class KernelTimer:
 
     def time_options(self, librecom_path: str, members: Sequence[int], num_options: int,
                      rounds: int = 3, repeats: int = 3, warmup: int = 4, tile_bytes: int = 0,
-                     xcd_segments: int = 0) -> List[List[float]]:
+                     xcd_segments: int = 0, only: Sequence[int] = None, seed: int = 0) -> List[List[float]]:
         """A library that holds ``num_options`` candidates for each feature in ``members`` (and one
         for every other feature): the whole kernel's time, summed over the batches, with all
-        members on option 0, all on option 1, ...  The options take turns ``rounds`` times, so
-        that a drift of the clocks meets all of them alike; returns the ``rounds`` times (ns) of
-        each option."""
-        import torch
-        from recflex_amd.rec_modules import FeatEmbed
-        layer = FeatEmbed(self.dev, embed_tables=self.tables, librecom=librecom_path)
-        counts = layer.lib.candidate_counts
+        members on option 0, all on option 1, ...  The options take turns ``rounds`` times in an
+        order drawn anew for every round, so that neither a drift of the clocks nor a place in
+        the order favours one of them; returns the ``rounds`` times (ns) of each option (``only``:
+        of these options, the others get an empty list)."""
+        from recflex_amd.librecom import RecomLib
+        counts = RecomLib(librecom_path).candidate_counts
         for f in members:
             if counts[f] != num_options:
                 raise ValueError(f"feature {f} holds {counts[f]} candidates, expected {num_options}")
+        todo = list(range(num_options)) if only is None else list(only)
+        mixes = []
+        for k in todo:
+            c = np.zeros(len(counts), dtype=np.int32)
+            c[list(members)] = k
+            mixes.append(c)
+        measured = self.time_mixes(librecom_path, mixes, rounds=rounds, repeats=repeats, warmup=warmup,
+                                   tile_bytes=tile_bytes, xcd_segments=xcd_segments, seed=seed)
+        times: List[List[float]] = [[] for _ in range(num_options)]
+        for k, t in zip(todo, measured):
+            times[k] = t
+        return times
+
+    def time_mixes(self, librecom_path: str, mixes: Sequence[np.ndarray], rounds: int = 3,
+                   repeats: int = 3, warmup: int = 4, tile_bytes: int = 0, xcd_segments: int = 0,
+                   seed: int = 0) -> List[List[float]]:
+        """The whole kernel's time (ns, summed over the batches) of a library that holds several
+        candidates per feature, for each of ``mixes`` (one candidate number per feature).  The
+        mixes take turns ``rounds`` times, in an order drawn anew for every round."""
+        import torch
+        from recflex_amd.rec_modules import FeatEmbed
+        layer = FeatEmbed(self.dev, embed_tables=self.tables, librecom=librecom_path)
         if self.outs is None:
             self.outs = [layer.forward_indices(d_idx, d_off).clone() for d_idx, d_off in self.batches]
         bound = [layer.bind_inputs(d_idx, d_off) for d_idx, d_off in self.batches]
-        choices = []
-        for k in range(num_options):
-            c = np.zeros(len(counts), dtype=np.int32)
-            c[list(members)] = k
-            choices.append(torch.from_numpy(c).to(self.dev))
-        times: List[List[float]] = [[] for _ in range(num_options)]
-        for r in range(rounds):
-            for k in range(num_options):
+        choices = [torch.from_numpy(np.asarray(c, dtype=np.int32)).to(self.dev) for c in mixes]
+        rng = np.random.default_rng(seed)
+        times: List[List[float]] = [[] for _ in mixes]
+        for choice in choices:                             # every mix warmed up once
+            for b, out in zip(bound, self.outs):
+                for _ in range(warmup):
+                    layer.forward_indices(b, out=out, tile_bytes=tile_bytes, xcd_segments=xcd_segments,
+                                          schedule_choice=choice)
+        for _ in range(rounds):
+            for k in rng.permutation(len(choices)):
                 total = 0.0
                 for b, out in zip(bound, self.outs):
                     run = lambda: layer.forward_indices(b, out=out, tile_bytes=tile_bytes,
                                                         xcd_segments=xcd_segments,
-                                                        schedule_choice=choices[k])
-                    for _ in range(warmup if r == 0 else 1):
-                        run()
+                                                        schedule_choice=choices[int(k)])
+                    run()
                     total += _timed_launches(run, repeats)
-                times[k].append(total)
+                times[int(k)].append(total)
         return times
 
 

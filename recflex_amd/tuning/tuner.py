@@ -94,10 +94,15 @@ class TuneConfig(NamedTuple):
     # the whole kernel is timed with the cluster on each of them in turn and the cluster adopts
     # the fastest if it beats its current pick by ``cluster_min_gain``.  ``cluster_sweeps`` passes
     # over all clusters, heaviest first, ``num_processes`` builds at a time.
+    # A scan over the options is followed by a head-to-head of the fastest against the current
+    # pick (the fastest of nine noisy times looks better than it is), and the adoptions of one
+    # group of builds -- all made against the same mix -- are then checked together in one more
+    # build, old picks against new, and dropped if the new mix is not faster.
     cluster_stage: bool = True
     cluster_top_k: int = 8
-    cluster_min_gain: float = 0.004
+    cluster_min_gain: float = 0.005
     cluster_sweeps: int = 1
+    cluster_group: int = 8
     # in-model local stage: compile every distinct candidate body alone for each occupancy and
     # keep out of that occupancy's tournament the ones that spill or come within
     # ``census_margin`` vector registers of the occupancy's budget (they cannot win, and their
@@ -128,6 +133,10 @@ class TuneConfig(NamedTuple):
     # global stage: also time the untuned default schedules at every occupancy and keep them
     # if they win (tile times measured feature by feature do not always add up to kernel time)
     include_default: bool = True
+    # global stage: a schedule file of an earlier tuning run of the same model (``schedule.json``
+    # as ``solve`` writes it), timed as one more contender at every occupancy: a model that is
+    # tuned again starts from what it has
+    incumbent: Optional[str] = None
 
 
 def padded_sched_num(orig_num: int, max_concurrent_blocks: int) -> int:
@@ -642,8 +651,26 @@ class Tuner:
         clusters = self.feature_clusters()
         timer = KernelTimer(self.table_shapes, self.data_types, self.data_npzs,
                             gpu_id=tune_config.gpu_ids[0])
-        width = max(1, tune_config.num_processes)
+        width = max(1, min(tune_config.num_processes, tune_config.cluster_group))
         log = []
+        checks = []
+
+        def emit_build(out: str, cands: list, note: dict) -> Optional[Tuple[str, str]]:
+            """Emit a production-shaped build holding ``cands``; the job to schedule, if any."""
+            if self._kept(out, tune_config) and os.path.exists(f"{out}/options.json"):
+                return None
+            os.makedirs(f"{out}/build", exist_ok=True)
+            emitter = CodeEmitter(None, feat_candidates=cands)
+            emitter.emit(f"{out}/process.hip", occupancy=occupancy, inline=tune_config.inline,
+                         tune=True, tile_bytes=tune_config.tile_bytes)
+            emitter.emit_cmake_list(f"{out}/CMakeLists.txt", code_fname="process.hip",
+                                    host_fname=None, subdirs=self.basic.subdirs,
+                                    includes=self.basic.includes, links=self.basic.links,
+                                    debug=tune_config.debug)
+            with open(f"{out}/options.json", "w") as f:
+                json.dump(note, f)
+            return out, f"{out}/build"
+
         for sweep in range(tune_config.cluster_sweeps):
             changed = False
             for lo in range(0, len(clusters), width):
@@ -660,44 +687,83 @@ class Tuner:
                     for f in members:
                         cands[f] += [self.feat_sched_param_candidates[f][k] for k in options]
                     out = self.get_cluster_dir(occupancy, sweep, ci)
-                    if not self._kept(out, tune_config) or not os.path.exists(f"{out}/options.json"):
-                        os.makedirs(f"{out}/build", exist_ok=True)
-                        emitter = CodeEmitter(None, feat_candidates=cands)
-                        emitter.emit(f"{out}/process.hip", occupancy=occupancy, inline=tune_config.inline,
-                                     tune=True, tile_bytes=tune_config.tile_bytes)
-                        emitter.emit_cmake_list(f"{out}/CMakeLists.txt", code_fname="process.hip",
-                                                host_fname=None, subdirs=self.basic.subdirs,
-                                                includes=self.basic.includes, links=self.basic.links,
-                                                debug=tune_config.debug)
-                        with open(f"{out}/options.json", "w") as f:
-                            json.dump({"members": members, "options": options,
-                                       "picks": [picks[f] for f in members]}, f)
-                        jobs.append((out, f"{out}/build"))
+                    job = emit_build(out, cands, {"members": members, "options": options,
+                                                  "picks": [picks[f] for f in members]})
+                    if job:
+                        jobs.append(job)
                     builds.append((ci, members, options, out))
                 self._schedule_builds(jobs, tune_config)
+                wanted = []                                   # (members, new pick, log entry)
                 for ci, members, options, out in builds:
-                    times = timer.time_options(f"{out}/build/librecom.so", members, len(options) + 1,
-                                               xcd_segments=DEFAULT_XCD_SEGMENTS)
+                    lib = f"{out}/build/librecom.so"
+                    times = timer.time_options(lib, members, len(options) + 1,
+                                               xcd_segments=DEFAULT_XCD_SEGMENTS, seed=ci)
                     med = [float(np.median(t)) for t in times]
                     best = int(np.argmin(med))
+                    entry = {"sweep": sweep, "cluster": ci, "members": members, "options": options,
+                             "kept_picks": [picks[f] for f in members], "kernel_ns": med,
+                             "adopted": None, "head_to_head_ns": None}
+                    log.append(entry)
                     gain = 1.0 - med[best] / med[0]
-                    adopt = best > 0 and gain >= tune_config.cluster_min_gain
-                    log.append({"sweep": sweep, "cluster": ci, "members": members,
-                                "options": options, "kept_picks": [picks[f] for f in members],
-                                "kernel_ns": med, "adopted": options[best - 1] if adopt else None})
+                    confirmed = 0.0
+                    if best > 0 and gain >= tune_config.cluster_min_gain:
+                        # the scan's winner against the current pick, taking turns
+                        again = timer.time_options(lib, members, len(options) + 1, rounds=6, repeats=5,
+                                                   xcd_segments=DEFAULT_XCD_SEGMENTS, only=[0, best],
+                                                   seed=1000 + ci)
+                        t_kept, t_best = float(np.median(again[0])), float(np.median(again[best]))
+                        entry["head_to_head_ns"] = [t_kept, t_best]
+                        confirmed = 1.0 - t_best / t_kept
+                        if confirmed >= tune_config.cluster_min_gain:
+                            wanted.append((members, options[best - 1], entry))
                     print(f"[clusters {occupancy}] sweep {sweep} cluster {ci} ({len(members)} features, "
                           f"dim {self.metas[members[0]].embed_dim}): kept {med[0]:.0f} ns, best option "
-                          f"{med[best]:.0f} ns ({100 * gain:.2f} %)" + (" -> adopted" if adopt else ""),
+                          f"{med[best]:.0f} ns ({100 * gain:.2f} %)"
+                          + (f", head to head {100 * confirmed:.2f} %" if entry["head_to_head_ns"] else ""),
                           flush=True)
-                    if adopt:
+                if len(wanted) > 1:
+                    # the group's adoptions together, old picks against new, in one more build
+                    switching = [f for members, _, _ in wanted for f in members]
+                    cands = [[self.feat_sched_param_candidates[f][picks[f]]] for f in range(self.num_feats)]
+                    for members, k, _ in wanted:
                         for f in members:
-                            picks[f] = options[best - 1]
-                        changed = True
+                            cands[f].append(self.feat_sched_param_candidates[f][k])
+                    out = f"{self.get_cluster_dir(occupancy, sweep, lo)}_check"
+                    job = emit_build(out, cands, {"members": switching})
+                    self._schedule_builds([job] if job else [], tune_config)
+                    # ... in which the adoptions join one by one, largest head-to-head gain first,
+                    # each kept only if the kernel gets faster with it than without
+                    lib = f"{out}/build/librecom.so"
+                    wanted.sort(key=lambda w: w[2]["head_to_head_ns"][1] / w[2]["head_to_head_ns"][0])
+                    current = np.zeros(self.num_feats, dtype=np.int32)
+                    kept_now = []
+                    for j, (members, k, entry) in enumerate(wanted):
+                        trial = current.copy()
+                        trial[members] = 1
+                        both = timer.time_mixes(lib, [current, trial], rounds=6, repeats=5,
+                                                xcd_segments=DEFAULT_XCD_SEGMENTS, seed=2000 + lo + j)
+                        t_without, t_with = float(np.median(both[0])), float(np.median(both[1]))
+                        ok = t_with < t_without * (1.0 - tune_config.cluster_min_gain / 2)
+                        checks.append({"sweep": sweep, "first_cluster": lo, "cluster": entry["cluster"],
+                                       "joined_after": len(kept_now), "kernel_ns": [t_without, t_with],
+                                       "kept": bool(ok)})
+                        print(f"[clusters {occupancy}] sweep {sweep}: cluster {entry['cluster']} joining "
+                              f"{len(kept_now)} adoptions: {t_without:.0f} -> {t_with:.0f} ns: "
+                              f"{'kept' if ok else 'dropped'}", flush=True)
+                        if ok:
+                            current = trial
+                            kept_now.append((members, k, entry))
+                    wanted = kept_now
+                for members, k, entry in wanted:
+                    entry["adopted"] = k
+                    for f in members:
+                        picks[f] = k
+                    changed = True
             if not changed:
                 break
         os.makedirs(os.path.dirname(result_log), exist_ok=True)
         with open(result_log, "w") as f:
-            json.dump({"picks": picks, "start": start, "clusters": log}, f)
+            json.dump({"picks": picks, "start": start, "clusters": log, "group_checks": checks}, f)
         return picks
 
     def _nearest_admitted(self, feat_id: int, pick: int, admitted: List[int]) -> int:
@@ -741,6 +807,77 @@ class Tuner:
                 with open(f"{output_dir}/result.txt") as f:     # absent if the worker failed
                     results[feat_id][occupancy] = list(map(float, f.read().strip().split(' ')))
         return results
+
+    def cluster_validation(self, occupancy: int, tune_config: TuneConfig) -> dict:
+        """Do the cluster stage's whole-kernel times in its candidate-holding builds carry over to
+        kernels built as they ship?  For every cluster of the first sweep (after
+        ``cluster_stage``: reads ``clusters/o{occ}/result.json``) the production kernel of the
+        mix the cluster was measured against is built with and without the cluster's fastest
+        option, both are timed taking turns, and the change is set beside the one the cluster
+        build showed.  Writes and returns ``clusters/o{occ}/validation.json``: per cluster the two
+        relative changes, and their Spearman rank correlation.  (The cluster-wise counterpart of
+        ``mutation_validation``.)"""
+        root = f"{self.basic.codegen_dir}/clusters/o{occupancy}"
+        with open(f"{root}/result.json") as f:
+            doc = json.load(f)
+        picks = list(doc["start"])
+        rows, jobs, mixes = [], [], {}
+
+        def production(name: str, mix_picks: List[int]) -> str:
+            out = f"{root}/validation/{name}"
+            mix = [self.feat_sched_param_candidates[f][k] for f, k in enumerate(mix_picks)]
+            if self._build_full(out, mix, occupancy, tune_config):
+                jobs.append((out, f"{out}/build"))
+            return f"{out}/build/librecom.so"
+
+        for entry in doc["clusters"]:
+            if entry["sweep"] != 0:
+                break
+            ns = entry["kernel_ns"]
+            best = int(np.argmin(ns[1:])) + 1 if len(ns) > 1 else 0
+            if best > 0:
+                swapped = list(picks)
+                for f in entry["members"]:
+                    swapped[f] = entry["options"][best - 1]
+                key = hashlib.sha256(json.dumps(picks).encode()).hexdigest()[:10]
+                mixes.setdefault(key, production(f"base_{key}", picks))
+                rows.append({"cluster": entry["cluster"], "members": entry["members"],
+                             "option": entry["options"][best - 1],
+                             "cluster_build_change": ns[best] / ns[0] - 1.0,
+                             "base": mixes[key], "swapped": production(f"c{entry['cluster']}", swapped)})
+            if entry["adopted"] is not None:
+                for f in entry["members"]:
+                    picks[f] = entry["adopted"]
+        self._schedule_builds(jobs, tune_config)
+        timer = KernelTimer(self.table_shapes, self.data_types, self.data_npzs,
+                            gpu_id=tune_config.gpu_ids[0])
+        for row in rows:
+            base, swapped = [], []
+            for _ in range(5):                                  # taking turns
+                base.append(timer.time_ns(row["base"], xcd_segments=DEFAULT_XCD_SEGMENTS, repeats=5))
+                swapped.append(timer.time_ns(row["swapped"], xcd_segments=DEFAULT_XCD_SEGMENTS, repeats=5))
+            row["production_ns"] = [float(np.median(base)), float(np.median(swapped))]
+            row["production_change"] = row["production_ns"][1] / row["production_ns"][0] - 1.0
+            del row["base"], row["swapped"]
+            print(f"[cluster validation {occupancy}] cluster {row['cluster']}: cluster build "
+                  f"{100 * row['cluster_build_change']:+.2f} %, production {100 * row['production_change']:+.2f} %",
+                  flush=True)
+
+        def ranks(v):
+            order = np.argsort(v, kind="stable")
+            r = np.empty(len(v))
+            r[order] = np.arange(len(v))
+            return r
+        rho = None
+        if len(rows) >= 3:
+            a = ranks([r["cluster_build_change"] for r in rows])
+            b = ranks([r["production_change"] for r in rows])
+            rho = float(np.corrcoef(a, b)[0, 1])
+        out = {"occupancy": occupancy, "rows": rows, "spearman": rho}
+        with open(f"{root}/validation.json", "w") as f:
+            json.dump(out, f, indent=1)
+        print(f"[cluster validation {occupancy}] {len(rows)} clusters, Spearman rank correlation {rho}", flush=True)
+        return out
 
     # ------------------------------------------------------------------ global stage
 
@@ -896,6 +1033,16 @@ class Tuner:
         for occupancy, sched_params in zip(tune_config.occupancies, occu_opt_sched_params):
             contenders.append((self.get_output_build_dir(-1, occupancy)[0], occupancy, sched_params))
         contenders += self.default_contenders(tune_config)
+        if tune_config.incumbent:
+            from recflex_amd.schedules import schedule_from_config
+            with open(tune_config.incumbent) as f:
+                doc = json.load(f)
+            entries = doc["schedules"] if isinstance(doc, dict) else doc
+            if len(entries) != self.num_feats:
+                raise ValueError(f"{tune_config.incumbent} describes {len(entries)} features, the model has {self.num_feats}")
+            mix = [schedule_from_config(e, meta, self.basic.block_threads) for e, meta in zip(entries, self.metas)]
+            for occupancy in tune_config.occupancies:
+                contenders.append((f"{self.basic.codegen_dir}/incumbent/o{occupancy}", occupancy, mix))
 
         jobs = []
         for output_dir, occupancy, sched_params in contenders:
@@ -921,7 +1068,7 @@ class Tuner:
             times.append(float(np.min(per_opt)))
             k = pick_launch_option(launch_opts, per_opt, tune_config.launch_time_tolerance)
             best_opts.append(launch_opts[k])
-            kind = "default" if "/default/o" in output_dir else "tuned"
+            kind = "default" if "/default/o" in output_dir else ("incumbent" if "/incumbent/o" in output_dir else "tuned")
             print(f"occupancy: {occupancy} ({kind}), t(ns): {times[-1]}"
                   + (f", (tile_bytes, xcd_segments): {launch_opts[k]} (of "
                      f"{ {o: round(t) for o, t in zip(launch_opts, per_opt)} })" if len(launch_opts) > 1 else ""))

@@ -455,28 +455,87 @@ def test_cluster_stage_adopts_by_whole_kernel_time(tmp_path, monkeypatch):
     asked = []
 
     class FakeTimer:
+        """Feature 4's option 2 (candidate 2) is 10 % faster in the scan and head to head; features
+        2 and 3 see 0.2 %, below the minimum gain; features 0 and 1 see an option win the scan
+        by 3 % that loses head to head (the fastest of several noisy times)."""
         def __init__(self, *a, **k):
             pass
 
-        def time_options(self, lib, members, num_options, **kw):
-            asked.append((tuple(members), num_options))
+        def time_options(self, lib, members, num_options, only=None, **kw):
+            asked.append((tuple(members), num_options, tuple(only) if only else None))
             base = [[100.0] * 3 for _ in range(num_options)]
             if tuple(members) == (4,):
-                base[2] = [90.0, 91.0, 89.0]                   # option 2 (candidate 2): 10 % faster
+                base[2] = [90.0, 91.0, 89.0]
             if tuple(members) == (2, 3):
-                base[1] = [99.8, 99.9, 99.7]                   # 0.2 %: below the minimum gain
+                base[1] = [99.8, 99.9, 99.7]
+            if tuple(members) == (0, 1):
+                base[3] = [97.0] * 3 if only is None else [100.2] * 3
             return base
 
     monkeypatch.setattr(tuner_mod, "KernelTimer", FakeTimer)
     start = [t._nearest_admitted(f, k, list(range(n))) for f, k in enumerate(t.default_choices()[0])]
     picks = t.cluster_stage(4, measured, tc)
-    assert asked == [((4,), 4), ((2, 3), 4), ((0, 1), 4)]
+    assert asked == [((4,), 4, None), ((4,), 4, (0, 2)), ((2, 3), 4, None), ((0, 1), 4, None),
+                     ((0, 1), 4, (0, 3))]
     assert picks[4] == 2 and picks[:4] == start[:4]
     doc = json.load(open(tmp_path / "out" / "clusters" / "o4" / "result.json"))
     assert doc["picks"] == picks and [c["adopted"] for c in doc["clusters"]] == [2, None, None]
+    assert doc["clusters"][2]["head_to_head_ns"] == [100.0, 100.2] and doc["group_checks"] == []
     # a second call reads the result file
     monkeypatch.setattr(tuner_mod, "KernelTimer", None)
     assert t.cluster_stage(4, measured, tc) == picks
+
+
+def test_cluster_adoptions_of_one_group_are_checked_together(tmp_path, monkeypatch):
+    """Two clusters of one group each win their head-to-head against the same old mix; in one
+    more build, old picks against new, they join one by one, the larger gain first -- and the
+    second, which makes the kernel slower once the first is in, is dropped."""
+    import recflex_amd.tuning.tuner as tuner_mod
+    rng = np.random.default_rng(4)
+    data = []
+    for f in range(3):
+        mean = [30, 30, 300][f]
+        bl = []
+        for _ in range(2):
+            lens = rng.poisson(mean, 16)
+            off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            bl.append((rng.integers(0, 100, off[-1]).astype(np.int32), off))
+        data.append(bl)
+    cfg = BasicConfig("", [], "", "", str(tmp_path / "out"), block_threads=256, sample_batch_nums=2)
+    t = Tuner(cfg, SCHEDULE_MAPPING, batches=data, table_shapes=[(100, 16)] * 3, data_types=["float"] * 3,
+              schedule_types=[[WarpPerSampleSchedule]] * 3)
+    n = len(t.feat_sched_param_candidates[0])
+    tc = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=4, in_process=True,
+                    register_census=False, cluster_top_k=2, cluster_min_gain=0.01)
+    scores = np.full(n, 10.0)
+    scores[[5, 2]] = [1.0, 2.0]
+    measured = {f: {4: scores.tolist()} for f in range(3)}
+    monkeypatch.setattr(Tuner, "_schedule_builds", lambda self, jobs, cfg_: None)
+    monkeypatch.setattr(Tuner, "_kept", lambda self, out, cfg_: False)
+
+    class FakeTimer:
+        def __init__(self, *a, **k):
+            pass
+
+        def time_options(self, lib, members, num_options, only=None, **kw):
+            base = [[100.0] * 3 for _ in range(num_options)]
+            base[1] = [95.0] * 3 if tuple(members) == (2,) else [97.0] * 3
+            return base
+
+        def time_mixes(self, lib, mixes, **kw):                # the group check: old against new
+            def t(mix):
+                mix = list(mix)
+                return {(0, 0, 0): 100.0, (0, 0, 1): 95.0, (1, 1, 1): 96.0}[tuple(mix)]
+            return [[t(m)] * 3 for m in mixes]
+
+    monkeypatch.setattr(tuner_mod, "KernelTimer", FakeTimer)
+    start = [t._nearest_admitted(f, k, list(range(n))) for f, k in enumerate(t.default_choices()[0])]
+    picks = t.cluster_stage(4, measured, tc)
+    doc = json.load(open(tmp_path / "out" / "clusters" / "o4" / "result.json"))
+    assert [(c["cluster"], c["joined_after"], c["kept"]) for c in doc["group_checks"]] == \
+        [(0, 0, True), (1, 1, False)]
+    assert picks[2] == 5 and picks[:2] == start[:2]            # the 5 % gain stays, the 3 % one goes
+    assert [c["adopted"] for c in doc["clusters"]] == [5, None]
 
 
 def test_task_blocks_of_the_frozen_binding_see_the_grid(tmp_path):
