@@ -102,7 +102,7 @@ int recom_get_max_concurrent_blocks(int32_t *out);
  * feature (rounded up to 128); a library with outlier tiles adds its list of outliers and
  * their partial sums (entries * (36 + 16 * max dim) + 128 bytes; 4 096 entries up to 128
  * features, 16 384 beyond); a library that is bound once per launch (by default one of more
- * than 512 features) adds the table into which a one-workgroup kernel binds the model (12 bytes
+ * than 2048 features) adds the table into which a one-workgroup kernel binds the model (12 bytes
  * per feature).  Replaces the
  * extra-buffer sizes the reference's host preprocessors report per batch
  * (RecFlex/code_emitter/codegen.py:149-160, extra_buffer_offsets). */
@@ -185,12 +185,12 @@ typedef struct recom_process_args {
   void *d_workspace;
   int64_t workspace_bytes;
   /* hipEvent_t (created by the caller with timing enabled) or NULL.  When either is given, the
-   * fused kernel is launched with hipExtLaunchKernel and the events receive the begin and the end
-   * of that very dispatch -- the kernel's own duration, without the dispatch latency and the
-   * marker packets that a pair of hipEventRecord calls around the launch adds (about two
-   * microseconds, which matter for a kernel of ten).  Kernels launched ahead of the fused one
-   * (outlier search, once-per-launch binding) are outside the pair.  Not for use under stream
-   * capture.  The reference times with the profiler only (RecFlex/cuda_helper.py:33-51). */
+   * kernels are launched with hipExtLaunchKernel: start_event receives the begin of the call's
+   * first dispatch (the fused kernel, or the kernel launched ahead of it: outlier search,
+   * once-per-launch binding), stop_event the end of the fused kernel's -- the call's own
+   * duration on the device, without the dispatch latency and the marker packets that a pair of
+   * hipEventRecord calls around the call adds (about two microseconds, which matter for a kernel
+   * of ten).  Not for use under stream capture.  The reference times with the profiler only (RecFlex/cuda_helper.py:33-51). */
   void *start_event;
   void *stop_event;
 } recom_process_args;
@@ -201,7 +201,7 @@ typedef struct recom_process_args {
  * and FusedKnl (RecFlex/code_emitter/codegen.py:318-383).
  * Never allocates.  A library emitted with outlier tiles (recom_info.outliers) launches a small
  * kernel ahead that walks the offsets and lists the outlier bags in the workspace.
- * A library that is bound once per launch (by default one of more than 512 features)
+ * A library that is bound once per launch (by default one of more than 2048 features)
  * launches a one-workgroup kernel ahead of the fused one that binds the model for this batch
  * into a table in the workspace. */
 int recom_process(const recom_process_args *args);

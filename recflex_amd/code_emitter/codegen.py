@@ -49,15 +49,13 @@ INDEX_BYTES = 4
 # than tiles of wide-row features.
 LOOKUP_OVERHEAD_BYTES = 0
 # Models of more features than this are bound once per launch by a small kernel instead of by
-# every workgroup of the fused kernel (rfx::bind_once), unless the emitter is told otherwise.
-# Up to rfx::kBindKeepAddrs (512) features a workgroup's own binding also leaves every feature's
-# addresses in LDS for its tiles; beyond, a tile reads them from memory either way and the
-# per-workgroup binding is only repeated work -- a thousand workgroups asking for the same two
-# cache lines per feature.  Measured on models of 256-bag batches of small features at four
-# workgroups per CU (per workgroup -> once per launch): 600 features 75.3 -> 72.0 us, 800
-# features 75.4 -> 70.6, 1 000 features 80.8 -> 75.1 (and 29.9 -> 28.8 at 300).  The
-# per-workgroup binding cannot hold more than 2 048 features in LDS beside four workgroups per CU.
-BIND_ONCE_MIN_FEATS = 512
+# every workgroup of the fused kernel (rfx::bind_once), unless the emitter is told otherwise
+# (``bind_once=``).  The per-workgroup binding cannot hold more than about 2 048 features in LDS
+# beside four workgroups per CU.  Below that the two ways cost the same for the whole call:
+# measured on models of 256-bag batches of small features at four workgroups per CU, back-to-back
+# launches from a graph, per workgroup -> once per launch: 1 000 features 81.5 -> 83.8 us (the
+# fused kernel alone 82.3 -> 76.1 us, the binding kernel 7.8 us and a launch in front of it).
+BIND_ONCE_MIN_FEATS = 2048
 # a bag becomes tiles of its own (libraries emitted with outliers=True) from this much traffic
 OUTLIER_MIN_BYTES = 128 * 1024
 
@@ -561,14 +559,24 @@ static int launch_kernels(const recom_process_args *a, void *workspace) {
   int stride_arg = static_cast<int>(row_stride);
   void *outlier_space = OUTLIERS ? static_cast<char *>(workspace) + SPLIT_BYTES : nullptr;
   void *bound = BIND_ONCE ? static_cast<char *>(workspace) + BOUND_OFFSET : nullptr;
+  // The caller's events take the begin of the call's first kernel and the end of its last
+  // (the fused kernel): a library that launches a kernel ahead of the fused one is timed whole.
+  hipStream_t stream = static_cast<hipStream_t>(a->stream);
+  hipEvent_t start_event = static_cast<hipEvent_t>(a->start_event);
+  hipEvent_t stop_event = static_cast<hipEvent_t>(a->stop_event);
+  auto launch = [&](const void *kernel, dim3 g, dim3 b, void **args, size_t lds, bool last) {
+    hipEvent_t s0 = start_event, s1 = last ? stop_event : nullptr;
+    start_event = nullptr;                                 // only the first kernel gets it
+    if (s0 || s1) return hipExtLaunchKernel(kernel, g, b, args, lds, stream, s0, s1, 0);
+    return hipLaunchKernel(kernel, g, b, args, lds, stream);
+  };
 #if RFX_OUTLIERS
   {
     void *outlier_args[] = {const_cast<int64_t **>(&a->d_io_ptrs), &arg_buffers,
                             const_cast<int64_t **>(&a->d_arg_buffer_offsets), &batch, &outlier_space};
     const unsigned gx = static_cast<unsigned>((batch + 255) / 256 > 64 ? 64 : (batch + 255) / 256);
     const unsigned gy = static_cast<unsigned>(NUM_FEATS > 1024 ? 1024 : NUM_FEATS);
-    e = hipLaunchKernel(reinterpret_cast<const void *>(OutlierKnl), dim3(gx, gy), dim3(256),
-                        outlier_args, 0, static_cast<hipStream_t>(a->stream));
+    e = launch(reinterpret_cast<const void *>(OutlierKnl), dim3(gx, gy), dim3(256), outlier_args, 0, false);
     if (e != hipSuccess) return static_cast<int>(e);
   }
 #endif
@@ -577,8 +585,7 @@ static int launch_kernels(const recom_process_args *a, void *workspace) {
   void *bind_args[] = {const_cast<int64_t **>(&a->d_io_ptrs), &arg_buffers,
                        const_cast<int64_t **>(&a->d_arg_buffer_offsets), &batch, &tile_arg,
                        const_cast<int32_t **>(&a->d_schedule_choice), &grid_arg, &bound};
-  e = hipLaunchKernel(reinterpret_cast<const void *>(BindKnl), dim3(1), dim3(1024), bind_args, 0,
-                      static_cast<hipStream_t>(a->stream));
+  e = launch(reinterpret_cast<const void *>(BindKnl), dim3(1), dim3(1024), bind_args, 0, false);
   if (e != hipSuccess) return static_cast<int>(e);
 #endif
   void *kernel_args[] = {
@@ -588,15 +595,8 @@ static int launch_kernels(const recom_process_args *a, void *workspace) {
       const_cast<int32_t **>(&a->d_schedule_choice),
       const_cast<unsigned long long **>(&a->d_times), &stride_arg, &bound, &workspace,
       &outlier_space};
-  if (a->start_event || a->stop_event)
-    // the events take the begin and end timestamps of this very dispatch
-    e = hipExtLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
-                           kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream),
-                           static_cast<hipEvent_t>(a->start_event),
-                           static_cast<hipEvent_t>(a->stop_event), 0);
-  else
-    e = hipLaunchKernel(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS),
-                        kernel_args, st->dyn_lds, static_cast<hipStream_t>(a->stream));
+  e = launch(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS), kernel_args,
+             st->dyn_lds, true);
   return static_cast<int>(e);
 }
 

@@ -35,14 +35,15 @@ its library is missing.  Names:
                    integer-valued tables, default schedules, emitted with outlier tiles;
                    ``c3_skew_plain``: the same without them
 ``fewbags``        8 fp32 features x 16 samples x 20 000 lookups, default schedules (split-bag);
-                   ``fewbags_unsplit``: the same with one workgroup per bag, for comparison
+                   ``fewbags_unsplit``: the same with one workgroup per bag, for comparison;
+                   ``fewbags64`` / ``fewbags128`` / ``fewbags512``: the same lookups as 64 x 4 000,
+                   128 x 2 500 and 512 x 1 000
 ``manysplit``      17 fp16 features of dim 256 under the split-bag schedule: 36 MB of workspace,
                    more than the static array of ``recom_process_static_workspace`` may hold
 ``refa``, ``reff4`` models shaped like the reference's example models A and a quarter of F (1 000 and
                    2 500 small features, batch 256; ``workloads.REF_SHAPED``), default schedules;
                    ``refa_tuned``: with ``tuned/refa_schedule.json`` if that file exists
-``wide``           1 500 small features, bound by every workgroup (``bind_once=False``: several
-                   binding rounds per thread)
+``wide``           1 500 small features (several binding rounds per thread)
 ``wider``          2 500 small features (bound once per launch by the binding kernel)
 """
 
@@ -247,11 +248,13 @@ def _c3_skew(outliers: bool) -> ModelSpec:
     return _default(wl, outliers=outliers)
 
 
-def _few_bags(split: bool) -> ModelSpec:
-    """Fewer bags than the device has workgroups, each of 20 000 lookups."""
-    feats = tuple(FeatureSpec(2_000_000, d, "float", 20000.0, False, 0.0, 1.0)
+def _few_bags(split: bool, bags: int = 16, lookups: float = 20000.0) -> ModelSpec:
+    """Fewer bags than the device has workgroups, each of ``lookups`` lookups (16 x 20 000 by
+    default; 64 x 4 000, 128 x 2 500 and 512 x 1 000 are the same eight features with the same
+    2.5 M lookups cut into more, shorter bags)."""
+    feats = tuple(FeatureSpec(2_000_000, d, "float", lookups, False, 0.0, 1.0)
                   for d in (32, 64, 128, 64, 32, 128, 64, 64))
-    wl = Workload("fewbags", 16, 77, feats, "integer")
+    wl = Workload("fewbags", bags, 77, feats, "integer")
     fs = default_feat_schedules(metas_of(wl), [f.mean_bag for f in feats], BLOCK_THREADS)
     assert all(isinstance(s, SplitBagSchedule) for s, _ in fs)
     if not split:
@@ -283,9 +286,7 @@ def _wide(num_features: int = 1500, name: str = "wide") -> ModelSpec:
         feats.append(FeatureSpec(int(rng.integers(64, 512)), dim, "float", mean, mean == 1.0,
                                  0.0 if mean == 1.0 else 0.3, 1.05))
     wl = Workload(name, 40, num_features, tuple(feats), "integer")
-    # wide: bound by every workgroup (several rounds of the binding loop per thread); wider: by
-    # the binding kernel
-    return _default(wl, bind_once=num_features > 2048)
+    return _default(wl)
 
 
 _SPECS: Dict[str, Callable[[], ModelSpec]] = {
@@ -323,6 +324,9 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c3_skew_plain": lambda: _c3_skew(False),
     "fewbags": lambda: _few_bags(True),
     "fewbags_unsplit": lambda: _few_bags(False),
+    "fewbags64": lambda: _few_bags(True, 64, 4000.0),
+    "fewbags128": lambda: _few_bags(True, 128, 2500.0),
+    "fewbags512": lambda: _few_bags(True, 512, 1000.0),
     "manysplit": _many_split,
     "wide": _wide,
     "wider": lambda: _wide(2500, "wider"),

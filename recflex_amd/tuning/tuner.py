@@ -103,6 +103,11 @@ class TuneConfig(NamedTuple):
     cluster_min_gain: float = 0.005
     cluster_sweeps: int = 1
     cluster_group: int = 8
+    # a cluster build is trusted only if it runs the current mix within this share of the time of
+    # the same mix built as it ships (heavy candidate bodies raise the registers and scratch of the
+    # kernel they sit in: an int8 model's cluster builds ran its default mix 40 % slower than
+    # its production build, and the options that won there lost 16 % in production)
+    cluster_build_tolerance: float = 0.05
     # in-model local stage: compile every distinct candidate body alone for each occupancy and
     # keep out of that occupancy's tournament the ones that spill or come within
     # ``census_margin`` vector registers of the occupancy's budget (they cannot win, and their
@@ -692,7 +697,14 @@ class Tuner:
                     if job:
                         jobs.append(job)
                     builds.append((ci, members, options, out))
+                # the mix as it is now, built as it ships: what a cluster build's own time with
+                # every cluster on its current pick has to come close to
+                base_out = f"{self.get_cluster_dir(occupancy, sweep, lo)}_base"
+                if self._build_full(base_out, [self.feat_sched_param_candidates[f][k]
+                                               for f, k in enumerate(picks)], occupancy, tune_config):
+                    jobs.append((base_out, f"{base_out}/build"))
                 self._schedule_builds(jobs, tune_config)
+                shipped_ns = timer.time_ns(f"{base_out}/build/librecom.so", xcd_segments=DEFAULT_XCD_SEGMENTS)
                 wanted = []                                   # (members, new pick, log entry)
                 for ci, members, options, out in builds:
                     lib = f"{out}/build/librecom.so"
@@ -702,10 +714,18 @@ class Tuner:
                     best = int(np.argmin(med))
                     entry = {"sweep": sweep, "cluster": ci, "members": members, "options": options,
                              "kept_picks": [picks[f] for f in members], "kernel_ns": med,
-                             "adopted": None, "head_to_head_ns": None}
+                             "shipped_ns": shipped_ns, "adopted": None, "head_to_head_ns": None}
                     log.append(entry)
                     gain = 1.0 - med[best] / med[0]
                     confirmed = 0.0
+                    if med[0] > shipped_ns * (1.0 + tune_config.cluster_build_tolerance):
+                        # the options' bodies change the kernel they sit in (registers, scratch):
+                        # what this build measures says nothing about the kernel that ships
+                        entry["unrepresentative"] = True
+                        print(f"[clusters {occupancy}] sweep {sweep} cluster {ci}: its build runs the "
+                              f"current mix in {med[0]:.0f} ns, the shipped build in {shipped_ns:.0f} ns: "
+                              f"not used", flush=True)
+                        continue
                     if best > 0 and gain >= tune_config.cluster_min_gain:
                         # the scan's winner against the current pick, taking turns
                         again = timer.time_options(lib, members, len(options) + 1, rounds=6, repeats=5,
@@ -743,6 +763,11 @@ class Tuner:
                         both = timer.time_mixes(lib, [current, trial], rounds=6, repeats=5,
                                                 xcd_segments=DEFAULT_XCD_SEGMENTS, seed=2000 + lo + j)
                         t_without, t_with = float(np.median(both[0])), float(np.median(both[1]))
+                        if j == 0 and t_without > shipped_ns * (1.0 + tune_config.cluster_build_tolerance):
+                            print(f"[clusters {occupancy}] sweep {sweep}: the check build runs the current "
+                                  f"mix in {t_without:.0f} ns, the shipped build in {shipped_ns:.0f} ns: "
+                                  f"nothing adopted", flush=True)
+                            break
                         ok = t_with < t_without * (1.0 - tune_config.cluster_min_gain / 2)
                         checks.append({"sweep": sweep, "first_cluster": lo, "cluster": entry["cluster"],
                                        "joined_after": len(kept_now), "kernel_ns": [t_without, t_with],

@@ -461,6 +461,9 @@ def test_cluster_stage_adopts_by_whole_kernel_time(tmp_path, monkeypatch):
         def __init__(self, *a, **k):
             pass
 
+        def time_ns(self, lib, **kw):                          # the mix built as it ships
+            return 100.0
+
         def time_options(self, lib, members, num_options, only=None, **kw):
             asked.append((tuple(members), num_options, tuple(only) if only else None))
             base = [[100.0] * 3 for _ in range(num_options)]
@@ -517,6 +520,9 @@ def test_cluster_adoptions_of_one_group_are_checked_together(tmp_path, monkeypat
         def __init__(self, *a, **k):
             pass
 
+        def time_ns(self, lib, **kw):
+            return 100.0
+
         def time_options(self, lib, members, num_options, only=None, **kw):
             base = [[100.0] * 3 for _ in range(num_options)]
             base[1] = [95.0] * 3 if tuple(members) == (2,) else [97.0] * 3
@@ -536,6 +542,37 @@ def test_cluster_adoptions_of_one_group_are_checked_together(tmp_path, monkeypat
         [(0, 0, True), (1, 1, False)]
     assert picks[2] == 5 and picks[:2] == start[:2]            # the 5 % gain stays, the 3 % one goes
     assert [c["adopted"] for c in doc["clusters"]] == [5, None]
+
+
+def test_cluster_build_that_is_not_like_the_shipped_build_is_not_used(tmp_path, monkeypatch):
+    """A cluster build that runs the current mix 40 % slower than the production build of that
+    mix (its candidates' bodies cost everybody registers) decides nothing, however good its
+    options look in it."""
+    import recflex_amd.tuning.tuner as tuner_mod
+    t = _tiny_tuner(tmp_path)
+    n0, n1 = (len(c) for c in t.feat_sched_param_candidates)
+    tc = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=2, in_process=True,
+                    register_census=False, cluster_top_k=2)
+    measured = {0: {4: list(np.arange(n0, 0, -1.0))}, 1: {4: list(np.arange(n1, 0, -1.0))}}
+    monkeypatch.setattr(Tuner, "_schedule_builds", lambda self, jobs, cfg_: None)
+    monkeypatch.setattr(Tuner, "_kept", lambda self, out, cfg_: False)
+
+    class FakeTimer:
+        def __init__(self, *a, **k):
+            pass
+
+        def time_ns(self, lib, **kw):
+            return 100.0
+
+        def time_options(self, lib, members, num_options, only=None, **kw):
+            return [[140.0] * 3] + [[110.0] * 3 for _ in range(num_options - 1)]
+
+    monkeypatch.setattr(tuner_mod, "KernelTimer", FakeTimer)
+    start = [t._nearest_admitted(f, k, list(range(len(t.feat_sched_param_candidates[f]))))
+             for f, k in enumerate(t.default_choices()[0])]
+    assert t.cluster_stage(4, measured, tc) == start
+    doc = json.load(open(tmp_path / "out" / "clusters" / "o4" / "result.json"))
+    assert all(c.get("unrepresentative") and c["adopted"] is None for c in doc["clusters"])
 
 
 def test_task_blocks_of_the_frozen_binding_see_the_grid(tmp_path):
