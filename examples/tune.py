@@ -83,7 +83,8 @@ def parse_args() -> argparse.Namespace:
                         help="emit the optimal library with outlier tiles: bags far longer than "
                              "their feature's schedule suits are found ahead of the fused kernel "
                              "and summed by several workgroups (for data with skewed bag lengths); "
-                             "auto = on if the sampled batches hold such a bag")
+                             "auto = if the sampled batches hold such a bag, the optimal mix is "
+                             "built both ways and timed on them, and the faster call is kept")
     parser.add_argument("--build_climb_trials", type=int, default=0,
                         help="global stage: that many single-feature variants of the winning mix are "
                              "built as production kernels and timed; the faster ones are adopted")

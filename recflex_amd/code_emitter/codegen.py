@@ -161,8 +161,7 @@ class CodeEmitter:
         its pair (-1 = none)."""
         thr, keys, body_of = [], [], []
         for cands in self.feat_candidates:
-            t = [schedule.LongBagThreshold(params) for schedule, params in cands]
-            t = 0 if min(t) <= 0 else max(t)
+            t = self._schedule_reach(cands)
             if t > 0:
                 per_lookup = cands[0][0].meta.row_bytes + INDEX_BYTES
                 t = max(t, -(-OUTLIER_MIN_BYTES // per_lookup))
@@ -172,6 +171,13 @@ class CodeEmitter:
                 keys.append(key)
             body_of.append(keys.index(key) if t > 0 else -1)
         return thr, keys, body_of
+
+    @staticmethod
+    def _schedule_reach(cands) -> int:
+        """The bag length beyond which the feature's schedule hands a bag to a whole wavefront
+        (0 = a schedule that handles long bags itself)."""
+        t = [schedule.LongBagThreshold(params) for schedule, params in cands]
+        return 0 if min(t) <= 0 else max(t)
 
     @staticmethod
     def _meta_of(dtype_id: int, dim: int):
@@ -283,13 +289,16 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
     char *__restrict__ {vars_.shmem}, rfx::f32x4 *__restrict__ {vars_.stage},
     const int {vars_.split_part}, const int {vars_.split_parts},
     float *__restrict__ {vars_.split_region}, const int {vars_.skip_long},
-    const int {vars_.one_per_bag}) {{
+    const int {vars_.one_per_bag}, rfx::MidBagQueue *{vars_.mid_queue}, const int {vars_.feat_id}) {{
+  (void){vars_.mid_queue}; (void){vars_.feat_id};
   {schedule.EmitScheduleBody(params)}
 }}
 '''
         # one block-wide body per (element type, dim) that can have outliers
-        long_cases = ""
+        long_cases, mid_cases = "", ""
         for k, (dtype_id, dim) in enumerate(long_keys):
+            mid_cases += (f"        case {k}: rfx::wave_bag<{dtype_id}, {dim}, {self.out_vec()}>"
+                          "(table, indices, beg, end, dst, lane); break;\n")
             meta = self._meta_of(dtype_id, dim)
             lanes = min(64, 1 << (meta.row_vectors - 1).bit_length())
             items = 4 if meta.elems_per_vector <= 4 else 2
@@ -374,7 +383,7 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
                      f"{vars_.bag_begin}, {vars_.bag_end}, reinterpret_cast<char *>(&s), "
                      + ("&s_stage.seg[0][0]" if need_stage else "nullptr")
                      + f", {vars_.split_part}, {vars_.split_parts}, {vars_.split_region}, {vars_.skip_long}"
-                     + f", {vars_.one_per_bag}")
+                     + f", {vars_.one_per_bag}, {vars_.mid_queue}, feat_idx")
         cases = "".join(
             f"      case {feat_idx}: ProcessFeat{feat_idx}({call_args}); break;\n"
             for feat_idx in body_ids)
@@ -422,17 +431,61 @@ extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
   rfx::find_outliers<NUM_FEATS>(d_outliers, io, c_long_thr, c_lookup_bytes);
 }
 ''' if outliers else ''
-        outlier_begin = '''
-  // outlier parts come first in the tile space: they are the longest tiles
+        outlier_begin = f'''
+  // the parts of the outlier bags of this batch (0: none, or more than the list holds)
   const int outlier_tiles = rfx::outlier_parts(d_outliers);
-  const int total_tiles = regular_tiles + outlier_tiles;
-''' if outliers else '''
-  constexpr int outlier_tiles = 0;
+  const int total_tiles = regular_tiles;
+  // mid-size bags wait here for a wavefront of this workgroup
+  __shared__ rfx::MidBagQueue s_mid_queue;
+  rfx::mid_queue_init<{vars_.BLOCK_THREADS}>(&s_mid_queue);
+  __syncthreads();
+  rfx::MidBagQueue *const {vars_.mid_queue} = &s_mid_queue;
+''' if outliers else f'''
   const int total_tiles = regular_tiles;
   (void)d_outliers;
+  rfx::MidBagQueue *const {vars_.mid_queue} = nullptr;
 '''
-        outlier_tile = f'''
-    if (tile < outlier_tiles) {{
+        drain_call = (f"if (rfx::mid_queue_pending({vars_.mid_queue})) DrainMidBags({vars_.mid_queue}, "
+                      f"d_embed_table_ptrs, io, d_output, {vars_.out_row_stride});")
+        # between its tiles a wavefront sums mid-size bags that wait in the workgroup's list
+        loop_tail = f"    {drain_call}\n" if outliers else ""
+        loop_head = '''  for (int walk = walk_first; walk < walk_last; walk += walk_step) {
+    int tile = walk;
+    if (by_xcd) {
+      const int seg = walk / seg_len;
+      tile = (seg * XCDS + xcd) * seg_len + (walk - seg * seg_len);
+      if (tile >= total_tiles) continue;
+    }
+'''
+        # Outlier parts are not dealt out with the regular tiles: a workgroup that has run its
+        # regular tiles draws parts from a ticket counter until none is left.  The next ticket is
+        # requested before the current part runs, so that its round trip is hidden behind the part.
+        # (Regular tiles held back and drawn the same way after the parts, to even out the end,
+        # were tried: a drawn tile needs the workgroup's wavefronts together, and with skewed bags
+        # each such tile waits for its slowest wavefront -- 191-210 us against 171.)
+        outlier_end = f'''
+  // A wavefront without regular tiles left takes mid-size bags until the last wavefront of the
+  // workgroup has finished its tiles and the list is empty.
+  rfx::mid_queue_walk_done({vars_.mid_queue});
+  for (;;) {{
+    const bool open = rfx::mid_queue_open({vars_.mid_queue});
+    if (rfx::mid_queue_pending({vars_.mid_queue}))
+      DrainMidBags({vars_.mid_queue}, d_embed_table_ptrs, io, d_output, {vars_.out_row_stride});
+    else if (!open)
+      break;
+    else
+      __builtin_amdgcn_s_sleep(8);
+  }}
+  if (outlier_tiles > 0) {{
+    __shared__ int s_ticket[2];
+    int slot = 0;
+    if (threadIdx.x == 0) s_ticket[0] = rfx::draw_outlier_part(d_outliers);
+    for (;;) {{
+      __syncthreads();
+      const int tile = s_ticket[slot];
+      if (tile >= outlier_tiles) break;
+      int next = 0;
+      if (threadIdx.x == 0) next = rfx::draw_outlier_part(d_outliers);
       const int entry = d_outliers->partmap[tile];
       const rfx::OutlierEntry e = d_outliers->entries[entry];
       const int part = tile - e.first;
@@ -441,15 +494,34 @@ extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
       const int *offsets = io.offsets(e.feat);
       const int embed_dim_offset = c_embed_dim_offsets[e.feat];
       switch (c_long_body[e.feat]) {{
-{long_cases}        default: break;
+{long_cases.replace(chr(10) + "  ", chr(10))}        default: break;
       }}
-      continue;
+      slot ^= 1;
+      if (threadIdx.x == 0) s_ticket[slot] = next;
     }}
-    tile -= outlier_tiles;
-''' if outliers else ''
-        outlier_end = '''
+  }}
   __syncthreads();
   if (threadIdx.x == 0) rfx::outliers_done(d_outliers);
+''' if outliers else ''
+        drain_func = f'''
+// Sums mid-size bags from the workgroup's list for as long as the calling wavefront gets one.
+__device__ __noinline__ void DrainMidBags(
+    rfx::MidBagQueue *q, const int64_t *__restrict__ d_embed_table_ptrs, const rfx::IoView io,
+    float *__restrict__ d_output, const int out_row_stride) {{
+  const int lane = threadIdx.x & 63;
+  int feat = 0, bag = 0;
+  while (rfx::mid_queue_pop(q, &feat, &bag)) {{
+    const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[feat]);
+    const int *indices = io.indices(feat);
+    const int *offsets = io.offsets(feat);
+    const int beg = __builtin_amdgcn_readfirstlane(offsets[bag]);
+    const int end = __builtin_amdgcn_readfirstlane(offsets[bag + 1]);
+    float *dst = d_output + static_cast<int64_t>(bag) * out_row_stride + c_embed_dim_offsets[feat];
+    switch (c_long_body[feat]) {{
+{mid_cases}      default: break;
+    }}
+  }}
+}}
 ''' if outliers else ''
         # rfx::kBindKeepAddrs: the binding of a model of up to 512 features keeps every feature's
         # table / indices / offsets address in LDS, and whether the batch holds one lookup per bag
@@ -464,7 +536,7 @@ extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
     const int *offsets = io.offsets(feat_idx);
     const int {vars_.one_per_bag} = 0;
 '''
-        kernel = bind_kernel + outlier_kernel + f'''
+        kernel = bind_kernel + outlier_kernel + drain_func + f'''
 extern "C" __global__ void {launch_bounds} FusedKnl(
     const int64_t *__restrict__ d_embed_table_ptrs,
     const int64_t *__restrict__ d_io_ptrs,
@@ -498,14 +570,8 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     walk_last = seg_len * xcd_segments;
     walk_step = gridDim.x / XCDS;
   }}
-  for (int walk = walk_first; walk < walk_last; walk += walk_step) {{
-    int tile = walk;
-    if (by_xcd) {{
-      const int seg = walk / seg_len;
-      tile = (seg * XCDS + xcd) * seg_len + (walk - seg * seg_len);
-      if (tile >= total_tiles) continue;
-    }}
-{outlier_tile}{timing_begin if timing and timing_branch else ''}
+{loop_head}
+{timing_begin if timing and timing_branch else ''}
     const int feat_idx = __builtin_amdgcn_readfirstlane(rfx::find_feature_wave<NUM_FEATS>(s_bind.prefix, tile));
     const int bags_per_tile = {bound_src}bags_per_tile[feat_idx];
     int {vars_.bag_begin} = (tile - s_bind.prefix[feat_idx]) * bags_per_tile;
@@ -531,7 +597,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
 {cases}      default: break;
     }}
 {timing_end}
-  }}
+{loop_tail}  }}
 {timing_flush}{outlier_end}}}
 
 '''

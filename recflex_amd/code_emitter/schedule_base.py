@@ -122,6 +122,11 @@ class ScheduleVars(NamedTuple):
     split_part: str = "split_part"
     split_parts: str = "split_parts"
     split_region: str = "split_region"
+    # rfx::MidBagQueue * (null in a build without outlier tiles): where a team leaves a bag
+    # beyond its schedule's reach for whichever wavefront of the workgroup has time, under the
+    # feature's number feat_id
+    mid_queue: str = "mid_queue"
+    feat_id: str = "feat_id"
 
 
 class PreprocessVars(NamedTuple):

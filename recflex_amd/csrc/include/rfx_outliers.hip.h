@@ -1,19 +1,29 @@
-// Outlier bags given to many workgroups (optional part of the fused embedding kernel, for data
+// Long bags taken out of the teams' hands (optional part of the fused embedding kernel, for data
 // whose bag lengths are skewed).
 //
 // A bag far longer than its feature's schedule was chosen for keeps one team -- at best one
-// wavefront (rfx::wave_bag) -- busy long after the rest of the grid has finished.  A library
-// emitted with outliers=True launches find_outliers ahead of the fused kernel: it walks all
-// offsets of the batch, and every bag longer than its schedule's threshold
-// (rfx::long_bag_threshold) becomes an entry {feature, bag, first part, parts} of a list in the
-// caller's workspace, parts = its traffic / kOutlierUnit (1..kOutlierMaxParts; 128, 256 and
-// 512 KiB per part give 227, 219 and 234 us on a 100-feature model with lognormal bag lengths).  The fused
-// kernel runs the parts of all entries as its first tiles, each like a part of a split bag
-// (rfx::split_part: partial sums in a slot, arrival counter, the last one adds the slots in
-// part order and writes the output), and its teams leave those bags alone.  If the list
-// overflows (more than CAP bags or 4 * CAP parts) the launch falls back to the
-// wavefront path for all of them.  The workgroup that finishes last puts the list header back
-// to zero for the next launch.
+// wavefront (rfx::wave_bag) -- busy long after the rest of the grid has finished, and the
+// wavefront that meets it in the middle of its tiles falls behind the others of its workgroup.
+// A library emitted with outliers=True deals with such bags at two levels.
+//   * Outliers: find_outliers, launched ahead of the fused kernel, walks all offsets of the
+//     batch, and every bag longer than its feature's outlier threshold (beyond its schedule's
+//     reach, rfx::long_bag_threshold, and at least 128 KiB of traffic) becomes an entry
+//     {feature, bag, first part, parts} of a list in the caller's workspace, parts = its
+//     traffic / kOutlierUnit (1..kOutlierMaxParts; 128, 256 and 512 KiB per part give 227, 219
+//     and 234 us on a 100-feature model with lognormal bag lengths).  The teams of the fused
+//     kernel leave those bags alone.  When a workgroup has run its share of the regular tiles it
+//     draws parts from a ticket counter until none is left, so that the workgroups whose
+//     regular tiles were cheap take more of them (dealt out like the regular tiles, three parts
+//     of 10-30 us to one workgroup and one to another, the same model spent a third of the
+//     kernel in its tail: 224 us against 192 with the parts drawn).  A part runs like a part of
+//     a split bag (rfx::split_part: the workgroup sums its share, partial sums in a slot,
+//     arrival counter, the last one adds the slots in part order and writes the output).  If
+//     the list overflows (more than CAP bags or 4 * CAP parts) the launch does without it.
+//     The workgroup that finishes last puts the list header back to zero for the next launch.
+//   * Mid-size bags (beyond the schedule's reach, below the outlier threshold) are summed by one
+//     wavefront, but not necessarily the one that met them: it puts them on a list of its
+//     workgroup in LDS (MidQueue), and every wavefront of the workgroup takes bags from that
+//     list between its tiles, so that the four wavefronts of a workgroup finish together.
 //
 // Reference counterpart: the role of rbk::SparseSegmentReduce
 // (examples/csrc/include/reduce_by_key_kernel.cuh), load balance under skewed bag lengths.
@@ -31,7 +41,8 @@ struct OutlierHeader {
   unsigned long long pack;                   // entries << 32 | parts, both as reserved so far
   int finished;                              // workgroups of the fused kernel that are done
   int last_entries, last_parts;              // what the previous launch found (for the caller)
-  int pad[27];
+  int next_part;                             // ticket counter: the next part nobody has taken yet
+  int pad[26];
 };
 struct OutlierEntry {
   int feat, bag, first, parts;
@@ -75,7 +86,7 @@ find_outliers(Space *__restrict__ sp, const IoView &io,
   }
 }
 
-// What the fused kernel reads when it starts: the number of outlier parts to run as tiles, 0 if
+// What the fused kernel reads when it starts: the number of outlier parts to draw, 0 if
 // there are none or the list overflowed (then the teams sum every bag themselves).
 template <typename Space>
 __device__ __forceinline__ int outlier_parts(const Space *sp) {
@@ -83,6 +94,12 @@ __device__ __forceinline__ int outlier_parts(const Space *sp) {
       __hip_atomic_load(&sp->hdr.pack, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const unsigned long long entries = pack >> 32, parts = pack & 0xffffffffull;
   return entries <= Space::kCap && parts <= Space::kPartCap ? static_cast<int>(parts) : 0;
+}
+
+// The next outlier part for the calling workgroup (one thread draws); at or beyond
+// the number of parts when all are taken.
+template <typename Space> __device__ __forceinline__ int draw_outlier_part(Space *sp) {
+  return __hip_atomic_fetch_add(&sp->hdr.next_part, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Called by every workgroup of the fused kernel when it has run out of tiles (by one thread):
@@ -96,6 +113,7 @@ template <typename Space> __device__ __forceinline__ void outliers_done(Space *s
     sp->hdr.last_entries = static_cast<int>(pack >> 32);
     sp->hdr.last_parts = static_cast<int>(pack & 0xffffffffull);
     __hip_atomic_store(&sp->hdr.finished, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&sp->hdr.next_part, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __hip_atomic_store(&sp->hdr.pack, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }

@@ -22,6 +22,7 @@
 // vectors are kept in flight per lane.
 #pragma once
 #include "rfx_arrival.h"
+#include "rfx_mid_queue.h"
 #include "rfx_binding.hip.h"
 #include "rfx_crosslane.hip.h"
 #include "rfx_rows.hip.h"
@@ -56,6 +57,82 @@ template <int BT> __device__ __forceinline__ int body_thread_id() {
   asm volatile("" : "+v"(lane));
   return (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) & (BT / 64 - 1)) * 64 + (lane & 63);
 }
+
+// ---------------------------------------------------------------------------------------------
+// The workgroup's list of mid-size bags (rfx_mid_queue.h) in LDS: workgroup-scope atomics, and
+// one lane acting for its wavefront.
+// ---------------------------------------------------------------------------------------------
+struct LdsMem {
+  static __device__ __forceinline__ int fetch_add(int *p, int v) {
+    return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  static __device__ __forceinline__ int load(int *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  static __device__ __forceinline__ bool compare_exchange(int *p, int *expected, int desired) {
+    return __hip_atomic_compare_exchange_strong(p, expected, desired, __ATOMIC_RELAXED,
+                                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  static __device__ __forceinline__ void store_entry(unsigned long long *p, unsigned long long v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  static __device__ __forceinline__ unsigned long long load_entry(unsigned long long *p) {
+    return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  static __device__ __forceinline__ void release_add(int *p, int v) {
+    __hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  static __device__ __forceinline__ int acquire_load(int *p) {
+    return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+};
+
+constexpr int kMidQueueCap = 192;
+using MidBagQueue = MidQueue<kMidQueueCap>;
+
+// by all threads of the workgroup, before a barrier that precedes the first use
+template <int BT> __device__ __forceinline__ void mid_queue_init(MidBagQueue *q) {
+  for (int i = threadIdx.x; i < kMidQueueCap; i += BT) q->e[i] = MidBagQueue::kEmpty;
+  if (threadIdx.x == 0) {
+    q->count = 0;
+    q->taken = 0;
+    q->walking = BT / 64;
+  }
+}
+
+// Called by a whole wavefront with uniform arguments; false: the list is full.
+__device__ __forceinline__ bool mid_queue_push(MidBagQueue *q, const int feat, const int bag) {
+  int ok = 0;
+  if ((threadIdx.x & 63) == 0) ok = mid_queue_push_one<LdsMem>(q, feat, bag) ? 1 : 0;
+  return __builtin_amdgcn_readfirstlane(ok) != 0;
+}
+
+// Called by a whole wavefront; true: {feat, bag} is the calling wavefront's to sum.
+__device__ __forceinline__ bool mid_queue_pop(MidBagQueue *q, int *feat, int *bag) {
+  unsigned int lo = 0, hi = 0;
+  int got = 0;
+  if ((threadIdx.x & 63) == 0) {
+    unsigned long long v = 0;
+    got = mid_queue_pop_one<LdsMem>(q, &v) ? 1 : 0;
+    lo = static_cast<unsigned int>(v);
+    hi = static_cast<unsigned int>(v >> 32);
+  }
+  if (!__builtin_amdgcn_readfirstlane(got)) return false;
+  *bag = static_cast<int>(__builtin_amdgcn_readfirstlane(lo));
+  *feat = static_cast<int>(__builtin_amdgcn_readfirstlane(hi));
+  return true;
+}
+
+__device__ __forceinline__ bool mid_queue_pending(MidBagQueue *q) {
+  return mid_queue_pending<LdsMem>(q);
+}
+
+// The calling wavefront has run its last regular tile.
+__device__ __forceinline__ void mid_queue_walk_done(MidBagQueue *q) {
+  if ((threadIdx.x & 63) == 0) mid_queue_walk_done_one<LdsMem>(q);
+}
+
+__device__ __forceinline__ bool mid_queue_open(MidBagQueue *q) { return mid_queue_open<LdsMem>(q); }
 
 // ---------------------------------------------------------------------------------------------
 // wave_bag: one bag summed by a whole wavefront, whatever the feature's schedule -- the way out
@@ -179,7 +256,8 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
           const int *__restrict__ indices,
           const int *__restrict__ offsets, float *__restrict__ out, const int esum,
           const int col_off, const int bag_begin, const int bag_end,
-          const int skip_longer_than = 0x7fffffff) {
+          const int skip_longer_than = 0x7fffffff, MidBagQueue *mid_queue = nullptr,
+          const int feat = 0) {
   using R = Row<DT, D>;
   constexpr int T = X * Y;
   static_assert(T >= 1 && T <= 64 && (T & (T - 1)) == 0, "team must be a power of two <= 64");
@@ -231,6 +309,8 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
           const int src = __builtin_ctzll(pending);
           pending &= pending - 1;
           const int b = __builtin_amdgcn_readlane(bag0 + i, src);
+          // left to whichever wavefront of the workgroup has time, if there is such a list
+          if (mid_queue && mid_queue_push(mid_queue, feat, b)) continue;
           wave_bag<DT, D, OVEC>(table, indices, __builtin_amdgcn_readlane(beg[i], src),
                                 __builtin_amdgcn_readlane(end[i], src),
                                 out + static_cast<int64_t>(b) * esum + col_off, tid & 63);
@@ -242,11 +322,15 @@ team_bags(f32x4 *__restrict__ stage, const char *__restrict__ table,
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < UB; ++i)
-        if (end[i] - beg[i] > skip_longer_than) {
+      for (int i = 0; i < UB; ++i) {
+        const int len = end[i] - beg[i];
+        // beyond this schedule's reach: another wavefront may have time for it sooner
+        if (len > skip_longer_than ||
+            (mid_queue && len > kLong && mid_queue_push(mid_queue, feat, bag0 + i))) {
           done_mask |= 1 << i;
           end[i] = beg[i];
         }
+      }
     }
     int len_max = 0;
 #pragma unroll

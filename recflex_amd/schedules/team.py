@@ -111,7 +111,8 @@ class TeamScheduleBase(ScheduleBase):
                  {p.items_per_thread}, {p.bags_per_team}, {p.vectors_per_pass}, {v.out_vec}>(
       {v.stage},
       {v.embed_table}, {v.indices}, {v.offsets}, {v.output},
-      {v.out_row_stride}, {v.embed_dim_offset}, {v.bag_begin}, {v.bag_end}, {v.skip_long});
+      {v.out_row_stride}, {v.embed_dim_offset}, {v.bag_begin}, {v.bag_end}, {v.skip_long},
+      {v.mid_queue}, {v.feat_id});
 '''
 
     def LongBagThreshold(self, params: NamedTuple) -> int:

@@ -76,8 +76,11 @@ class TuneConfig(NamedTuple):
     tile_bytes: int = DEFAULT_TILE_BYTES
     # emit optimal/ with outlier tiles: bags far beyond their schedule's reach are found by a pass
     # over the offsets ahead of the fused kernel and summed by several workgroups (skewed data).
-    # None: decided from the sampled batches -- on if any of them holds such a bag
+    # None: decided on the sampled batches -- if any of them holds such a bag, the mix is built
+    # both ways and the faster call wins (Tuner.decide_outliers)
     outliers: Optional[bool] = None
+    # undecided (None): kept only if the whole call is faster by this share on the samples
+    outliers_min_gain: float = 0.02
     # local-stage interference: "model" = every candidate of every feature is compiled into one
     # kernel of the whole model and timed while all other features run beside it;
     # "replicate" = per feature, the candidates side by side over the same data, replicated
@@ -160,6 +163,20 @@ def pick_launch_option(launch_opts: List[Tuple[int, int]], times: List[float],
     limit = times[best] * (1.0 + tolerance)
     near = [k for k, (_, xs) in enumerate(launch_opts) if xs > 0 and times[k] <= limit]
     return min(near, key=lambda k: (launch_opts[k][1], times[k]))
+
+
+def release_device_memory() -> None:
+    """Hands the device memory that this process's earlier measurements left in torch's caching
+    allocator back to the driver.  The measurements that follow run in child processes, which
+    build the model's tables again: for a model whose tables fill most of the device (C4) the
+    child otherwise runs out of memory."""
+    import gc
+    import sys
+    gc.collect()
+    torch = sys.modules.get("torch")
+    if torch is not None and torch.cuda.is_initialized():
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
 
 
 class Tuner:
@@ -927,6 +944,42 @@ class Tuner:
                 return True
         return False
 
+    def decide_outliers(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
+                        tile_bytes: int, xcd_segments: int, tune_config: TuneConfig) -> bool:
+        """Outlier tiles on or off for ``optimal/``, by measurement: if a sampled batch holds a
+        bag that a library with outlier tiles would run as tiles of its own, the mix is built
+        both ways and timed on the samples like a contender of the global stage; outlier tiles
+        are kept if the whole call (the pass that finds the outliers included) is faster by
+        ``TuneConfig.outliers_min_gain``.  Such a bag alone does not decide: the list and the
+        arrival of the parts cost the fused kernel registers and LDS, and a model whose long bags
+        are a small share of its traffic loses more to that than the outliers cost it (C4: 10 %).
+        """
+        if not self.has_outlier_bags(sched_params):
+            print("outlier tiles: off (no sampled bag beyond its schedule's reach)", flush=True)
+            return False
+        dirs = {on: f"{self.basic.codegen_dir}/outliers_{'on' if on else 'off'}/o{occupancy}"
+                for on in (False, True)}
+        jobs = []
+        for on, output_dir in dirs.items():
+            self.emit_codes(output_dir=output_dir, feat_schedules=sched_params, occupancy=occupancy,
+                            inline=tune_config.inline, debug=tune_config.debug, tile_bytes=tile_bytes,
+                            xcd_segments=max(xcd_segments, 0), outliers=on)
+            jobs.append((output_dir, f"{output_dir}/build"))
+        self._schedule_builds(jobs, tune_config)
+        manager = self._measure_manager(tune_config)
+        if tune_config.profiler == "rocprofv3" or manager:
+            release_device_memory()
+        cfg = tune_config._replace(remeasure=True)
+        for output_dir in dirs.values():
+            self._kernel_time(output_dir, cfg, manager)
+        if manager:
+            manager.join()
+        t_off, t_on = (self._read_kernel_time(dirs[on], tune_config) for on in (False, True))
+        keep = t_on < t_off * (1.0 - tune_config.outliers_min_gain)
+        print(f"outlier tiles: {'on' if keep else 'off'} (measured on the sampled batches: "
+              f"{t_on:.0f} ns with, {t_off:.0f} ns without)", flush=True)
+        return keep
+
     def solve(self, measured_times: Dict[int, Dict[int, List[float]]],
               tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
         occu_opt_sched_params = self.select_per_occupancy(measured_times, tune_config.occupancies)
@@ -947,9 +1000,13 @@ class Tuner:
             print(f"occupancy: {opt_occupancy} (after the build climb), t(ns): {t}", flush=True)
         outliers = tune_config.outliers
         if outliers is None:
-            outliers = self.has_outlier_bags(opt_sched_params)
-            print(f"outlier tiles: {'on' if outliers else 'off'} (decided from the sampled batches)", flush=True)
-        if climbed or tile_bytes != tune_config.tile_bytes or xcd_segments or outliers:
+            outliers = self.decide_outliers(opt_sched_params, opt_occupancy, tile_bytes, xcd_segments,
+                                            tune_config)
+        # a contender whose library came out of the compile cache (the same source had been built
+        # in another directory) has no host module of its own: optimal/ is then built in place
+        import glob
+        host_missing = not glob.glob(f"{optimal}/build/recom_host*.so")
+        if climbed or tile_bytes != tune_config.tile_bytes or xcd_segments or outliers or host_missing:
             # make the winning launch parameters the defaults of the optimal library
             self.emit_codes(output_dir=optimal, feat_schedules=opt_sched_params, occupancy=opt_occupancy,
                             inline=tune_config.inline, debug=tune_config.debug, tile_bytes=tile_bytes,
@@ -1021,8 +1078,18 @@ class Tuner:
             # per batch the median over the measured passes of the call's kernels (the fused
             # kernel and what the library launches ahead of it), summed over the batches: the
             # same quantity the events timer reports
-            return float(sum(parse_knl_batch_times("FusedKnl", f"{report_prefix}_kernel_trace.csv",
-                                                   PROFILE_PASSES, PROFILE_WARMUP_PASSES)))
+            try:
+                return float(sum(parse_knl_batch_times("FusedKnl", f"{report_prefix}_kernel_trace.csv",
+                                                       PROFILE_PASSES, PROFILE_WARMUP_PASSES)))
+            except (ValueError, OSError) as e:
+                # say what the profiled child printed: the trace alone does not tell why it is short
+                log = f"{report_prefix}.rocprofv3.log"
+                tail = ""
+                if os.path.exists(log):
+                    with open(log, errors="replace") as f:
+                        tail = "".join(f.readlines()[-15:])
+                raise RuntimeError(f"no usable kernel trace for {output_dir} ({e}); the profiled "
+                                   f"run printed:\n{tail}") from e
         with open(f"{report_prefix}.events.txt") as f:
             return float(f.read().strip())
 
@@ -1078,6 +1145,8 @@ class Tuner:
         launch_opts = [(tb, xs) for tb in (list(tune_config.tile_bytes_candidates) or [0])
                        for xs in (list(tune_config.xcd_segments_candidates) or [0])]
         manager = self._measure_manager(tune_config)
+        if tune_config.profiler == "rocprofv3" or manager:
+            release_device_memory()
         for output_dir, occupancy, _ in contenders:
             for tile_bytes, xcd_segments in launch_opts:
                 self._kernel_time(output_dir, tune_config, manager, tile_bytes, xcd_segments)

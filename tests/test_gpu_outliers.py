@@ -28,12 +28,16 @@ def _inject(rng, wl, indices, offsets, plan):
     return indices, offsets
 
 
-@pytest.mark.parametrize("case", ["none", "few", "many", "overflow"])
+@pytest.mark.parametrize("case", ["none", "few", "many", "overflow", "mid", "mid_overflow"])
 def test_outlier_tiles_are_bit_exact(case):
     """No outlier at all; a few bags of 300 to 20 000 lookups in features of every kind of
     schedule; some hundred outliers; more than the list holds (4 096), where the launch falls back
-    to a wavefront per outlier.  Three launches each on one workspace, whose list header and
-    arrival counters must be back at zero afterwards.  Integer-valued tables: bit for bit."""
+    to a wavefront per outlier; some hundred mid-size bags (beyond their schedule's reach, below
+    the outlier threshold: they go through the workgroup's list in LDS to whichever wavefront
+    has time); every bag of twenty features mid-size, more than that list holds (192 per
+    workgroup), where a bag is summed by the wavefront that met it.  Three launches each on one
+    workspace, whose list header and arrival counters must be back at zero afterwards.
+    Integer-valued tables: bit for bit."""
     import torch
     from recflex_amd import prebuilt
     from recflex_amd.rec_modules import FeatEmbed
@@ -59,8 +63,12 @@ def test_outlier_tiles_are_bit_exact(case):
             plan = {int(f): [int(x)] for f, x in zip(feats[:6], (300, 2000, 20000, 4200, 5000, 9000))}
         elif case == "many":
             plan = {int(f): [2000 + 371 * k for k in range(12)] for f in feats[:10]}
-        else:
+        elif case == "overflow":
             plan = {int(f): 2500 for f in feats[:60]}
+        elif case == "mid":
+            plan = {int(f): [70 + 13 * k for k in range(40)] for f in feats[:12]}
+        else:
+            plan = {int(f): 90 + 7 * int(f) % 60 for f in feats[:20]}
         indices, offsets = _inject(rng, wl, base_idx, base_off, plan)
         d_idx = [torch.from_numpy(i).to(dev) for i in indices]
         d_off = [torch.from_numpy(o).to(dev) for o in offsets]
@@ -72,7 +80,7 @@ def test_outlier_tiles_are_bit_exact(case):
         # CAP entries of 4 ints, CAP counters, PARTS part -> entry, PARTS slots of 128 floats
         ws = layer.workspace.cpu().numpy()
         ws = ws[len(ws) - (32 + 4 * CAP + CAP + PARTS + PARTS * 128):]
-        assert not ws[:3].any(), f"launch {launch}: list header not cleared: {ws[:3].tolist()}"
+        assert not ws[:3].any() and not ws[5], f"launch {launch}: list header not cleared: {ws[:6].tolist()}"
         assert not ws[32 + 4 * CAP:32 + 5 * CAP].any(), f"launch {launch}: arrival counters not reset"
         # what the launch found: bags beyond their schedule's threshold and 128 KiB of traffic
         # (split-bag features take bags of any length themselves)
@@ -84,5 +92,5 @@ def test_outlier_tiles_are_bit_exact(case):
         assert int(ws[3]) == expect, (int(ws[3]), expect)
         if case == "overflow":
             assert expect > CAP
-        elif case != "none":
+        elif case in ("few", "many"):
             assert 0 < expect <= CAP and int(ws[4]) >= expect

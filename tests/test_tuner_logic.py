@@ -361,6 +361,34 @@ def test_outlier_tiles_are_switched_on_by_the_sampled_data():
     assert not tuner.has_outlier_bags(fs)
 
 
+def test_outlier_tiles_are_kept_only_if_the_call_is_faster(tmp_path, monkeypatch):
+    """An outlier bag in the samples makes the tuner build the mix with and without outlier tiles
+    and time both; the tiles stay only if the whole call gains ``outliers_min_gain``.  Without
+    such a bag nothing is built."""
+    tuner = _tiny_tuner(tmp_path)
+    mix = [c[0] for c in tuner.feat_sched_param_candidates]
+    built, times = [], {}
+    monkeypatch.setattr(Tuner, "_schedule_builds", lambda self, jobs, cfg: built.extend(j[0] for j in jobs))
+    monkeypatch.setattr(Tuner, "_kernel_time", lambda self, d, cfg, mgr, tb=0, xs=0: None)
+    monkeypatch.setattr(Tuner, "_read_kernel_time",
+                        lambda self, d, cfg, tb=0, xs=0: times["on" if "outliers_on" in d else "off"])
+    cfg = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=1, in_process=True,
+                     cluster_stage=False)
+    monkeypatch.setattr(Tuner, "has_outlier_bags", lambda self, sp: False)
+    assert tuner.decide_outliers(mix, 4, 65536, 16, cfg) is False and not built
+    monkeypatch.setattr(Tuner, "has_outlier_bags", lambda self, sp: True)
+    times.update(on=900.0, off=1000.0)
+    assert tuner.decide_outliers(mix, 4, 65536, 16, cfg) is True
+    assert len(built) == 2 and any("outliers_on" in d for d in built)
+    on_src = open([d for d in built if "outliers_on" in d][0] + "/process.hip").read()
+    off_src = open([d for d in built if "outliers_off" in d][0] + "/process.hip").read()
+    assert "find_outliers" in on_src and "find_outliers" not in off_src
+    times.update(on=990.0, off=1000.0)            # within the margin: not worth a second kernel
+    assert tuner.decide_outliers(mix, 4, 65536, 16, cfg) is False
+    times.update(on=1100.0, off=1000.0)           # C4's case
+    assert tuner.decide_outliers(mix, 4, 65536, 16, cfg) is False
+
+
 def test_kernel_trace_parser_groups_calls_and_takes_medians(tmp_path):
     """rocprofv3 ``*_kernel_trace.csv``: a call is a FusedKnl dispatch plus the library's own
     kernels launched ahead of it; per batch the median over the passes after the warm-up pass."""
