@@ -63,9 +63,10 @@ typedef struct recom_info {
   int32_t reserved[3];
 } recom_info;
 
-#define RECOM_ABI_VERSION 5     /* 4: recom_process_static_workspace; the once-per-launch binding
+#define RECOM_ABI_VERSION 6     /* 4: recom_process_static_workspace; the once-per-launch binding
                                  * table of very wide models moved into the workspace
-                                 * 5: recom_process_args.start_event / stop_event */
+                                 * 5: recom_process_args.start_event / stop_event
+                                 * 6: recom_process_args.d_lookup_counts */
 
 /* largest workspace recom_process_static_workspace serves from the library's static array */
 #define RECOM_STATIC_WORKSPACE_MAX_BYTES (32 * 1024 * 1024)
@@ -193,6 +194,14 @@ typedef struct recom_process_args {
    * of ten).  Not for use under stream capture.  The reference times with the profiler only (RecFlex/cuda_helper.py:33-51). */
   void *start_event;
   void *stop_event;
+  /* Optional hint for the run-time binding: device int32[F], the number of lookups of each
+   * feature in this batch as far as the caller knows (the length of its index array).  NULL: the
+   * binding reads offsets[batch] of every feature itself -- one scattered cache line per feature
+   * and workgroup, half of the binding's time for a model of a thousand features.  The figures
+   * only size the tiles (and tell the row-copy schedule that a feature may hold one lookup per
+   * bag, which it verifies bag by bag): a wrong figure costs balance, never correctness.  The
+   * reference has no counterpart (its binding runs on the host). */
+  const int32_t *d_lookup_counts;
 } recom_process_args;
 
 /* Launch the fused kernel: for every feature f and sample b,

@@ -412,9 +412,9 @@ extern "C" __global__ void __launch_bounds__(1024) BindKnl(
     const int64_t *__restrict__ d_io_ptrs, const char *__restrict__ d_arg_buffers,
     const int64_t *__restrict__ d_arg_buffer_offsets, const int batch, const int tile_bytes,
     const int *__restrict__ d_schedule_choice, const int grid_blocks,
-    rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound) {{
+    rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound, const int *__restrict__ d_lookup_counts) {{
   __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;
-  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
+  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch, d_lookup_counts}};
   rfx::bind_once<NUM_FEATS, 1024, HAS_SPLIT>(s_bind, d_bound, io, tile_bytes, c_lookup_bytes, c_bag_bytes,
                                   c_cand_begin, c_cand_gran, d_schedule_choice, {fixed_arg},
                                   grid_blocks);
@@ -547,11 +547,11 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     const int *__restrict__ d_schedule_choice,
     unsigned long long *__restrict__ d_times, const int {vars_.out_row_stride},
     const rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound, float *__restrict__ d_workspace,
-    OutlierSpace *__restrict__ d_outliers) {{
+    OutlierSpace *__restrict__ d_outliers, const int *__restrict__ d_lookup_counts) {{
 {bind_decl}
   __shared__ KnlTempStorage s;
 {stage_decl}{timing_init}
-  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch}};
+  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch, d_lookup_counts}};
 {bind_call}
 {timing_bound}
 {outlier_begin}
@@ -650,7 +650,8 @@ static int launch_kernels(const recom_process_args *a, void *workspace) {
   int grid_arg = grid;
   void *bind_args[] = {const_cast<int64_t **>(&a->d_io_ptrs), &arg_buffers,
                        const_cast<int64_t **>(&a->d_arg_buffer_offsets), &batch, &tile_arg,
-                       const_cast<int32_t **>(&a->d_schedule_choice), &grid_arg, &bound};
+                       const_cast<int32_t **>(&a->d_schedule_choice), &grid_arg, &bound,
+                       const_cast<int32_t **>(&a->d_lookup_counts)};
   e = launch(reinterpret_cast<const void *>(BindKnl), dim3(1), dim3(1024), bind_args, 0, false);
   if (e != hipSuccess) return static_cast<int>(e);
 #endif
@@ -660,7 +661,7 @@ static int launch_kernels(const recom_process_args *a, void *workspace) {
       const_cast<float **>(&a->d_output), &batch, &tile_arg, &xcd_arg,
       const_cast<int32_t **>(&a->d_schedule_choice),
       const_cast<unsigned long long **>(&a->d_times), &stride_arg, &bound, &workspace,
-      &outlier_space};
+      &outlier_space, const_cast<int32_t **>(&a->d_lookup_counts)};
   e = launch(reinterpret_cast<const void *>(FusedKnl), dim3(grid), dim3(BLOCK_THREADS), kernel_args,
              st->dyn_lds, true);
   return static_cast<int>(e);

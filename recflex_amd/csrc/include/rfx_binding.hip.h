@@ -38,6 +38,9 @@ struct IoView {
   const char *__restrict__ arg_base;
   const int64_t *__restrict__ arg_offsets;
   int batch;
+  // optional: the lookups of every feature in this batch as the caller knows them (a hint for
+  // the binding, which otherwise reads offsets[batch] of every feature)
+  const int *__restrict__ counts = nullptr;
 
   __device__ __forceinline__ int64_t offsets_addr(int f) const {
     if (io_ptrs) return io_ptrs[2 * f + 1];
@@ -259,9 +262,15 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     cost[k] = 0;
     bool one_per_bag = false;
     if (!fixed_tiles) {
-      const int *offs = global_ptr<int>(offs_at[k]);
-      const int first_lookup = offs[0];
-      const int64_t lookups = static_cast<int64_t>(offs[B]) - first_lookup;
+      int first_lookup = 0;
+      int64_t lookups;
+      if (io.counts) {                        // one array for all features instead of a line each
+        lookups = io.counts[f];
+      } else {
+        const int *offs = global_ptr<int>(offs_at[k]);
+        first_lookup = offs[0];
+        lookups = static_cast<int64_t>(offs[B]) - first_lookup;
+      }
       cost[k] = lookups * lookup_b[k] + static_cast<int64_t>(B) * bag_b[k];
       traffic += real ? static_cast<float>(cost[k]) : 0.f;
       one_per_bag = lookups == B && first_lookup == 0;

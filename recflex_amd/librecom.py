@@ -61,10 +61,11 @@ class RecomProcessArgs(ctypes.Structure):
         ("workspace_bytes", ctypes.c_int64),
         ("start_event", ctypes.c_void_p),
         ("stop_event", ctypes.c_void_p),
+        ("d_lookup_counts", ctypes.c_void_p),
     ]
 
 
-RECOM_ABI_VERSION = 5
+RECOM_ABI_VERSION = 6
 RECOM_STATIC_WORKSPACE_MAX_BYTES = 32 * 1024 * 1024
 RECOM_ESTATIC_WORKSPACE = -5
 EXPORTED_SYMBOLS = ("recom_get_info", "recom_get_feature_tables", "recom_get_candidate_counts",
@@ -175,11 +176,14 @@ class RecomLib:
                 grid_blocks: int = 0, xcd_segments: int = 0, schedule_choice: int = 0,
                 times: int = 0, stream: int = 0, output_row_stride: int = 0,
                 workspace: int = 0, workspace_bytes: int = 0,
-                static_workspace: bool = False, start_event: int = 0, stop_event: int = 0) -> None:
+                static_workspace: bool = False, start_event: int = 0, stop_event: int = 0,
+                lookup_counts: int = 0) -> None:
         """All pointer arguments are raw device addresses (``tensor.data_ptr()``).  Without a
         ``workspace``, a library that needs one uses ``default_workspace()``.
         ``start_event`` / ``stop_event``: ``hipEvent_t`` handles that receive the begin and end of
         the fused kernel's own dispatch.
+        ``lookup_counts``: device int32[F], the lookups of each feature in this batch as far as
+        the caller knows (a hint that spares the binding a scattered read per feature).
         ``static_workspace=True`` calls ``recom_process_static_workspace`` instead: no workspace
         is passed or allocated, the library uses its own static device array."""
         if static_workspace:
@@ -187,7 +191,7 @@ class RecomLib:
                                     arg_buffer_offsets or None, output or None, batch, tile_bytes,
                                     grid_blocks, xcd_segments, schedule_choice or None,
                                     times or None, stream or None, output_row_stride, None, 0,
-                                    start_event or None, stop_event or None)
+                                    start_event or None, stop_event or None, lookup_counts or None)
             rc = self.lib.recom_process_static_workspace(ctypes.byref(args))
             if rc == RECOM_ESTATIC_WORKSPACE:
                 raise RecomError(f"recom_process_static_workspace: the library needs "
@@ -202,7 +206,8 @@ class RecomLib:
                                 arg_buffer_offsets or None, output or None, batch, tile_bytes,
                                 grid_blocks, xcd_segments, schedule_choice or None, times or None,
                                 stream or None, output_row_stride, workspace or None,
-                                workspace_bytes, start_event or None, stop_event or None)
+                                workspace_bytes, start_event or None, stop_event or None,
+                                lookup_counts or None)
         rc = self.lib.recom_process(ctypes.byref(args))
         if rc != 0:
             raise RecomError("recom_process", rc)

@@ -60,9 +60,13 @@ def default_feat_schedules(metas: Sequence[MetaData], mean_bag_lens: Sequence[fl
             for m, l, h in zip(metas, mean_bag_lens, one_hot)]
 
 
+def feat_schedules_from_entries(entries: Sequence[dict], block_threads: int = 256) -> FeatSchedules:
+    """The schedules that ``CodeEmitter.serialize_config`` wrote as a list of entries."""
+    return [schedule_from_config(e, MetaData(e["embed_dim"], e.get("data_type", "float")), block_threads)
+            for e in entries]
+
+
 def load_feat_schedules(schedule_json: str, block_threads: int = 256) -> FeatSchedules:
     """Read back what ``CodeEmitter.dump_key`` / ``serialize_config`` wrote."""
     with open(schedule_json) as f:
-        entries = json.load(f)
-    return [schedule_from_config(e, MetaData(e["embed_dim"], e.get("data_type", "float")), block_threads)
-            for e in entries]
+        return feat_schedules_from_entries(json.load(f), block_threads)

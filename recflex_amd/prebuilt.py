@@ -54,7 +54,7 @@ from typing import Callable, Dict, List, NamedTuple, Optional
 import numpy as np
 
 from .code_emitter import MetaData
-from .model_build import FeatSchedules, build_model, default_feat_schedules, load_feat_schedules
+from .model_build import FeatSchedules, build_model, default_feat_schedules, feat_schedules_from_entries
 from .schedules import (BlockPerBagSchedule, SplitBagSchedule, SubWavefrontPerBagSchedule,
                         ThreadPerBagSchedule, WavefrontPerBagSchedule)
 from .workloads import FeatureSpec, Workload, make_workload
@@ -102,12 +102,7 @@ def _tuned(wl: Workload, fname: str) -> ModelSpec:
         doc = json.load(f)
     entries = doc["schedules"] if isinstance(doc, dict) else doc
     occupancy = doc.get("occupancy") if isinstance(doc, dict) else None
-    tmp = os.path.join(MODELS_DIR, f".{fname}.entries.json")
-    os.makedirs(MODELS_DIR, exist_ok=True)
-    with open(tmp, "w") as f:
-        json.dump(entries, f)
-    fs = load_feat_schedules(tmp, BLOCK_THREADS)
-    os.remove(tmp)
+    fs = feat_schedules_from_entries(entries, BLOCK_THREADS)
     assert len(fs) == wl.num_features
     kwargs = {}
     if isinstance(doc, dict) and doc.get("tile_bytes"):

@@ -253,7 +253,11 @@ class FeatEmbed(nn.Module):
         flat[0::2] = [t.data_ptr() for t in indices]
         flat[1::2] = [t.data_ptr() for t in offsets]
         io_ptrs = torch.tensor(flat, dtype=torch.int64, device=self.device)
-        return BoundInputs(batch, io_ptrs, (list(indices), list(offsets)))
+        # the lengths of the index arrays: a hint that spares the kernel's binding one scattered
+        # read per feature (recom_process_args.d_lookup_counts; wrong figures -- tensors refilled
+        # with fewer lookups than they hold -- cost balance only)
+        counts = torch.tensor([t.numel() for t in indices], dtype=torch.int32, device=self.device)
+        return BoundInputs(batch, io_ptrs, (list(indices), list(offsets)), counts)
 
     def check_inputs(self, indices: Sequence[torch.Tensor], offsets: Sequence[torch.Tensor]) -> None:
         """Debugging aid: raise ``ValueError`` if a launch on these inputs would read outside a
@@ -305,7 +309,9 @@ class FeatEmbed(nn.Module):
         batch = bound.batch
         res = self._launch(batch, timing, timing_schedules, tile_bytes, grid_blocks,
                            schedule_choice=schedule_choice, out=out, xcd_segments=xcd_segments,
-                           kernel_events=kernel_events, io_ptrs=bound.io_ptrs.data_ptr())
+                           kernel_events=kernel_events, io_ptrs=bound.io_ptrs.data_ptr(),
+                           lookup_counts=(bound.lookup_counts.data_ptr()
+                                          if bound.lookup_counts is not None else 0))
         if timing:
             return res[0].view(batch, self.output_units), res[1]
         return res.view(batch, self.output_units)
@@ -316,6 +322,7 @@ class BoundInputs(NamedTuple):
     batch: int
     io_ptrs: torch.Tensor       # int64 [2 * F] on the device: indices_f, offsets_f addresses
     tensors: tuple              # keeps the bound tensors alive
+    lookup_counts: Optional[torch.Tensor] = None    # int32 [F] on the device: len(indices_f)
 
 
 class FeatProcessEmbed(nn.Module):

@@ -56,7 +56,8 @@ def test_ctypes_structs_match_header_layout():
     # recom_info: 11 named int32 + 5 reserved; recom_process_args: 5 pointers, 4 int32,
     # 3 pointers, an int64, a pointer and an int64 on LP64
     assert ctypes.sizeof(RecomInfo) == 16 * 4
-    assert ctypes.sizeof(RecomProcessArgs) == 5 * 8 + 4 * 4 + 3 * 8 + 8 + 8 + 8 + 2 * 8
+    assert ctypes.sizeof(RecomProcessArgs) == 5 * 8 + 4 * 4 + 3 * 8 + 8 + 8 + 8 + 2 * 8 + 8
+    assert RecomProcessArgs.d_lookup_counts.offset == 120
     assert RecomProcessArgs.output_row_stride.offset == 80
     assert RecomProcessArgs.d_workspace.offset == 88 and RecomProcessArgs.workspace_bytes.offset == 96
     assert RecomProcessArgs.start_event.offset == 104 and RecomProcessArgs.stop_event.offset == 112

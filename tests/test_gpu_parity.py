@@ -273,6 +273,39 @@ def test_row_copy_template_on_any_input(case, batch):
     assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
 
 
+@pytest.mark.parametrize("name", ["onehots", "c3s_outliers", "fewbags128"])
+def test_lookup_count_hint_sizes_tiles_and_nothing_else(name):
+    """``recom_process_args.d_lookup_counts``: the binding takes the lookups per feature from the
+    caller instead of reading ``offsets[batch]`` of every feature.  Right figures (what
+    ``bind_inputs`` passes), none, and wrong ones -- all zero, all equal to the batch (which tells
+    the row-copy schedule that every bag has one lookup), ten times too many -- give the same
+    output: bit for bit on integer-valued tables, also where the figures change how a split bag
+    is cut into parts."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    wl = prebuilt.model_spec(name).workload
+    assert wl.table_values == "integer"
+    dev = torch.device("cuda", 0)
+    print(f"[case] {name}: lookup-count hint", flush=True)
+    tables = gen_tables(wl, dev)
+    indices, offsets = gen_inputs(wl)
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib(name))
+    bound = layer.bind_inputs([torch.from_numpy(i).to(dev) for i in indices],
+                              [torch.from_numpy(o).to(dev) for o in offsets])
+    assert bound.lookup_counts.cpu().tolist() == [len(i) for i in indices]
+    want = oracle_output(wl, [t.cpu().numpy() for t in tables], indices, offsets)
+    true = bound.lookup_counts
+    variants = {"right": true, "none": None, "zero": torch.zeros_like(true),
+                "one_per_bag": torch.full_like(true, wl.batch), "tenfold": true * 10}
+    for label, counts in variants.items():
+        got = layer.forward_indices(bound._replace(lookup_counts=counts)).cpu().numpy()
+        bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+        assert bad.size == 0, f"{label}: {len(bad)} elements differ, first at {bad[:5].tolist()}"
+
+
 def test_gather_probe_runs():
     """The measurement aid of bench.py: fetches the rows of a batch and nothing else.  It must
     run to completion on ragged inputs (empty features, rows of 1 to 64 vectors) and take time."""
