@@ -659,16 +659,17 @@ class Tuner:
     def cluster_stage(self, occupancy: int, measured_times: Dict[int, Dict[int, List[float]]],
                       tune_config: TuneConfig) -> List[int]:
         """Second half of the in-model local stage (see ``TuneConfig.cluster_stage``).  Starts
-        from the default-heuristic mix (each pick moved to the nearest candidate the register
-        census admits at this occupancy); returns the index of every feature's pick in its
-        candidate list.  ``clusters/o{occ}/result.json`` keeps what was measured."""
+        from the default-heuristic mix as it is -- also where the register census keeps a
+        default pick out of this occupancy's tournament: the census judges a body alone, the
+        default mix is what a production build at this occupancy runs, and moving such a pick to
+        its nearest admitted neighbour made the start 20 % slower than the default on the int8
+        model.  Returns the index of every feature's pick in its candidate list.
+        ``clusters/o{occ}/result.json`` keeps what was measured."""
         result_log = f"{self.basic.codegen_dir}/clusters/o{occupancy}/result.json"
         if os.path.exists(result_log) and not tune_config.remeasure:
             with open(result_log) as f:
                 return json.load(f)["picks"]
-        admitted = self.admitted_candidates(occupancy)
-        picks = [admitted[f][self._nearest_admitted(f, k, admitted[f])]
-                 for f, k in enumerate(self.default_choices()[0])]
+        picks = [int(k) for k in self.default_choices()[0]]
         start = list(picks)
         clusters = self.feature_clusters()
         timer = KernelTimer(self.table_shapes, self.data_types, self.data_npzs,
