@@ -31,6 +31,8 @@ its library is missing.  Names:
 ``c3s_outliers``   c3s with integer-valued tables, emitted with ``outliers=True``: bags beyond a
                    schedule's threshold are found ahead of the kernel and run as tiles of their
                    own; every tenth feature under the split-bag schedule
+``c4s_outliers``, ``c5s_outliers``  c4s (fp16) and c5s (int8) with integer-valued tables and
+                   outlier tiles
 ``c3_skew``        C3 with bag lengths from a lognormal (sigma 1.5) of the same means and
                    integer-valued tables, default schedules, emitted with outlier tiles;
                    ``c3_skew_plain``: the same without them
@@ -314,6 +316,11 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     # by the binding kernel all the same (an emit option)
     "c3s_bind_once": lambda: _default(make_workload("C3", batch=192, max_rows=60_000), bind_once=True),
     "c3s_outliers": _c3s_outliers,
+    # fp16 and int8 tables with outlier tiles (integer-valued: sums exact)
+    "c4s_outliers": lambda: _default(make_workload("C4", batch=128, num_features=48, max_rows=30_000)
+                                     ._replace(name="c4s_outliers", table_values="integer"), outliers=True),
+    "c5s_outliers": lambda: _default(make_workload("C5", batch=256, num_features=24, max_rows=50_000)
+                                     ._replace(name="c5s_outliers", table_values="integer"), outliers=True),
     "variants": _variants,
     "edge": _edge,
     "onehots": _onehots,

@@ -94,3 +94,40 @@ def test_outlier_tiles_are_bit_exact(case):
             assert expect > CAP
         elif case in ("few", "many"):
             assert 0 < expect <= CAP and int(ws[4]) >= expect
+
+
+@pytest.mark.parametrize("name", ["c4s_outliers", "c5s_outliers"])
+@pytest.mark.parametrize("case", ["few", "mid"])
+def test_outlier_tiles_on_fp16_and_int8_rows(name, case):
+    """The block-wide parts, the workgroup's list of mid-size bags and the wavefront that sums
+    them, on fp16 and int8 rows (scale and bias, staged output): a few bags of 300 to 20 000
+    lookups, and some hundred bags between their schedule's reach and the outlier threshold.
+    Two launches on one workspace; integer-valued tables, bit for bit."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    spec = prebuilt.model_spec(name)
+    wl = spec.workload
+    assert wl.table_values == "integer"
+    dev = torch.device("cuda", 0)
+    print(f"[case] {name} {case}: F={wl.num_features} B={wl.batch}", flush=True)
+    tables = gen_tables(wl, dev)
+    host_tables = [t.cpu().numpy() for t in tables]
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib(name))
+    assert layer.lib.info.outliers == 1 and layer.workspace is not None
+    rng = np.random.default_rng(len(name) + len(case))
+    base_idx, base_off = gen_inputs(wl)
+    for launch in range(2):
+        feats = rng.permutation(wl.num_features)
+        if case == "few":
+            plan = {int(f): [int(x)] for f, x in zip(feats[:6], (300, 2000, 20000, 4200, 5000, 9000))}
+        else:
+            plan = {int(f): [70 + 13 * k for k in range(30)] for f in feats[:8]}
+        indices, offsets = _inject(rng, wl, base_idx, base_off, plan)
+        got = layer.forward_indices([torch.from_numpy(i).to(dev) for i in indices],
+                                    [torch.from_numpy(o).to(dev) for o in offsets]).cpu().numpy()
+        want = oracle_output(wl, host_tables, indices, offsets)
+        bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+        assert bad.size == 0, f"launch {launch}: {len(bad)} elements differ, first at {bad[:5].tolist()}"
