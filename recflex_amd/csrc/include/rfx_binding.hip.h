@@ -72,9 +72,9 @@ struct IoView {
 // a granularity of kSplitGran.  A bag is worth splitting when it alone would keep its workgroup
 // busy for a good part of the kernel: the unit is a quarter of a workgroup's fair share of the
 // batch's traffic (total / grid), at least one tile and kSplitMinUnit; when the mean bag of such a feature
-// carries more than two units, the feature gets batch * parts tiles, parts = bag / unit, tile t
+// carries more than 1.25 units, the feature gets batch * parts tiles, parts = bag / unit, tile t
 // being part t % parts of bag t / parts, and bags_per_tile holds -parts.  (A part costs some
-// 20 us of dependent memory round trips besides its rows, and with two to five tiles per
+// 6 us of dependent memory round trips besides its rows, and with two to five tiles per
 // workgroup the time moves in steps of whole tiles: a unit of half a share gave 150 / 162 /
 // 161 us where a quarter gives 177 / 109 / 160 us on 16 x 20 000, 64 x 4 000 and 128 x 2 500
 // lookups; the finer one is kept, it also evens out bags of unequal length.)
