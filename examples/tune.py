@@ -85,6 +85,12 @@ def parse_args() -> argparse.Namespace:
                              "and summed by several workgroups (for data with skewed bag lengths); "
                              "auto = if the sampled batches hold such a bag, the optimal mix is "
                              "built both ways and timed on them, and the faster call is kept")
+    parser.add_argument("--walk_stage", choices=["auto", "on", "off"], default="auto",
+                        help="after the global stage, try the winning mix with its features laid out in "
+                             "the tile space by their time per tile, and with the last passes of the "
+                             "tile walk drawn from ticket counters, and keep what is faster on the "
+                             "samples; auto = for models of 256 features and more whose workgroups get fewer "
+                             "than eight tiles each")
     parser.add_argument("--build_climb_trials", type=int, default=0,
                         help="global stage: that many single-feature variants of the winning mix are "
                              "built as production kernels and timed; the faster ones are adopted")
@@ -182,7 +188,8 @@ def create_tune_config(args: argparse.Namespace) -> TuneConfig:
               "cluster_sweeps": args.cluster_sweeps, "incumbent": args.incumbent,
               "build_climb_trials": args.build_climb_trials,
               "build_climb_top_k": args.build_climb_top_k,
-              "climb_passes": args.climb_passes, "outliers": {"auto": None, "on": True, "off": False}[args.outliers]}
+              "climb_passes": args.climb_passes, "outliers": {"auto": None, "on": True, "off": False}[args.outliers],
+              "walk_stage": {"auto": None, "on": True, "off": False}[args.walk_stage]}
     if args.tile_bytes:
         kwargs["tile_bytes"] = args.tile_bytes
     if args.xcd_segments_candidates:

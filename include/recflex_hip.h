@@ -102,7 +102,8 @@ int recom_get_max_concurrent_blocks(int32_t *out);
  * schedule that splits bags over workgroups, then 2048 * (D_f + 1) * 4 bytes for each such
  * feature (rounded up to 128); a library with outlier tiles adds its list of outliers and
  * their partial sums (entries * (36 + 16 * max dim) + 128 bytes; 4 096 entries up to 128
- * features, 16 384 beyond); a library that is bound once per launch (by default one of more
+ * features, 16 384 beyond); a library whose last tile passes are drawn from ticket counters
+ * adds those (1 152 bytes); a library that is bound once per launch (by default one of more
  * than 2048 features) adds the table into which a one-workgroup kernel binds the model (12 bytes
  * per feature).  Replaces the
  * extra-buffer sizes the reference's host preprocessors report per batch
@@ -175,7 +176,8 @@ typedef struct recom_process_args {
    * (the kernel then stores 16 bytes at a time), and d_output aligned likewise. */
   int64_t output_row_stride;
   /* Workspace of the schedules that give one bag to several workgroups (batches of few, very
-   * long bags), of the outlier tiles and of the once-per-launch binding of very wide models:
+   * long bags), of the outlier tiles, of a drawn end of the tile walk and of the once-per-launch
+   * binding of very wide models:
    * device memory of at least recom_get_workspace_bytes() bytes, 16-byte aligned,
    * caller allocated.  It must be all zero before the first launch that uses it; every launch
    * leaves its arrival counters at zero again, so it is cleared once, not per launch.  Launches

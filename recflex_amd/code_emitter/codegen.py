@@ -210,7 +210,8 @@ class CodeEmitter:
                     timing_branch: bool = False, fixed_task_block_nums: List[int] = None,
                     tile_bytes: int = None, xcd_aware: bool = False,
                     lookup_overhead_bytes: int = None, xcd_segments: int = 8,
-                    outliers: bool = False, bind_once: bool = None) -> str:
+                    outliers: bool = False, bind_once: bool = None,
+                    tile_order: List[int] = None, drawn_tail: int = 0) -> str:
         num_feats = len(self.feat_schedules)
         if lookup_overhead_bytes is None:
             lookup_overhead_bytes = LOOKUP_OVERHEAD_BYTES
@@ -230,6 +231,25 @@ class CodeEmitter:
         assert not outliers or all(len(c) == 1 for c in self.feat_candidates)
         long_thr, long_keys, long_body_of = self.long_bag_tables() if outliers else ([], [], [])
         outliers = outliers and len(long_keys) > 0
+        # Tile order: place p of the kernel's tile space holds feature tile_order[p] of the model.
+        # Inside the kernel a feature's number is its place: every per-feature table below is
+        # emitted in that order, and what the caller passes per feature is found through
+        # c_ext_feat (rfx::IoView::ext).  Everything the library says about itself to the host
+        # (recom_get_feature_tables ...) stays in the model's order.
+        if tile_order is not None:
+            tile_order = [int(f) for f in tile_order]
+            assert sorted(tile_order) == list(range(num_feats)), "tile_order must be a permutation of the features"
+            assert all(len(c) == 1 for c in self.feat_candidates) and not timing and not fixed_task_block_nums, \
+                "a tile order goes with a production build (one schedule per feature, no timers, no frozen binding)"
+            if tile_order == list(range(num_feats)):
+                tile_order = None
+
+        def placed(per_feature: list) -> list:
+            return [per_feature[f] for f in tile_order] if tile_order is not None else list(per_feature)
+        # the last passes of the tile walk drawn from ticket counters (rfx::TailTickets) instead
+        # of dealt out: a production option, and the outlier tiles have their own drawn end
+        assert not (drawn_tail and (outliers or timing or fixed_task_block_nums)), \
+            "drawn_tail goes with neither outlier tiles nor timers nor a frozen binding"
         max_long_dim = max([(d + 3) // 4 * 4 for _, d in long_keys], default=4)
         fixed_arg = "c_fixed_task_block_nums" if fixed_task_block_nums else "nullptr"
 
@@ -256,8 +276,13 @@ constexpr bool HAS_SPLIT = SPLIT_BYTES > 0;
 #define RFX_OUTLIERS {1 if outliers else 0}
 constexpr bool OUTLIERS = RFX_OUTLIERS;
 constexpr int MAX_LONG_DIM = {max_long_dim};
-using OutlierSpace = rfx::OutlierSpace<MAX_LONG_DIM, {outlier_capacity(num_feats)}>;
-constexpr long long OUTLIER_BYTES = OUTLIERS ? (long long)sizeof(OutlierSpace) : 0LL;
+// ... or, in their place in the workspace, the ticket counters of a drawn end of the tile walk
+#define RFX_DRAWN_TAIL {int(drawn_tail)}
+constexpr int DRAWN_TAIL = RFX_DRAWN_TAIL;
+static_assert(!(OUTLIERS && DRAWN_TAIL > 0), "one or the other");
+using OutlierSpace = {"rfx::TailTickets" if drawn_tail else f"rfx::OutlierSpace<MAX_LONG_DIM, {outlier_capacity(num_feats)}>"};
+constexpr long long OUTLIER_BYTES = OUTLIERS || DRAWN_TAIL > 0 ? (long long)sizeof(OutlierSpace) : 0LL;
+#define RFX_TILE_ORDER {1 if tile_order is not None else 0}
 // the binding table of a model that is bound once per launch (rfx::bind_once) comes last
 constexpr long long BOUND_OFFSET = (SPLIT_BYTES + OUTLIER_BYTES + 255) / 256 * 256;
 constexpr long long BOUND_BYTES = BIND_ONCE ? (long long)sizeof(rfx::BoundTables<NUM_FEATS>) : 0LL;
@@ -315,20 +340,28 @@ __device__ {"__forceinline__" if inline else "__noinline__"} void ProcessFeat{fe
         temp_storage_decl += "};\n\n"
 
         tables = _c_array("int", "c_cand_begin", cand_begin)
-        tables += _c_array("int", "c_cand_func_ids", [id_map[i] for i in range(len(flat))])
-        tables += _c_array("int", "c_cand_gran", [s.TileGranularity(p) for s, p in flat])
-        tables += _c_array("int", "c_embed_dim_offsets", embed_dim_offsets)
+        if tile_order is not None:
+            # one candidate per feature: a candidate's number is its feature's
+            tables += _c_array("int", "c_cand_func_ids", placed([id_map[i] for i in range(len(flat))]))
+            tables += _c_array("int", "c_cand_gran", placed([s.TileGranularity(p) for s, p in flat]))
+            tables += _c_array("int", "c_ext_feat", tile_order)
+        else:
+            tables += _c_array("int", "c_cand_func_ids", [id_map[i] for i in range(len(flat))])
+            tables += _c_array("int", "c_cand_gran", [s.TileGranularity(p) for s, p in flat])
+        # first output column of every feature, and (last entry) the width of the output
+        tables += _c_array("int", "c_embed_dim_offsets", placed(embed_dim_offsets[:-1]) + [embed_dim_offsets[-1]])
+        tables += _c_array("int", "c_embed_dims", placed([s.meta.embed_dim for s, _ in self.feat_schedules]))
         tables += _c_array("int", "c_lookup_bytes",
-                           [s.meta.row_bytes + INDEX_BYTES + lookup_overhead_bytes
-                            for s, _ in self.feat_schedules])
+                           placed([s.meta.row_bytes + INDEX_BYTES + lookup_overhead_bytes
+                                   for s, _ in self.feat_schedules]))
         tables += _c_array("int", "c_bag_bytes",
-                           [s.meta.embed_dim * 4 + BAG_FIXED_BYTES for s, _ in self.feat_schedules])
+                           placed([s.meta.embed_dim * 4 + BAG_FIXED_BYTES for s, _ in self.feat_schedules]))
         if has_split:
             # first float of each feature's region of the workspace (-1: the feature has none)
-            tables += _c_array("long long", "c_split_region", split_regions)
+            tables += _c_array("long long", "c_split_region", placed(split_regions))
         if outliers:
-            tables += _c_array("int", "c_long_thr", long_thr)
-            tables += _c_array("int", "c_long_body", long_body_of)
+            tables += _c_array("int", "c_long_thr", placed(long_thr))
+            tables += _c_array("int", "c_long_body", placed(long_body_of))
         if fixed_task_block_nums:
             assert len(fixed_task_block_nums) == num_feats
             tables += _c_array("int", "c_fixed_task_block_nums",
@@ -414,22 +447,23 @@ extern "C" __global__ void __launch_bounds__(1024) BindKnl(
     const int *__restrict__ d_schedule_choice, const int grid_blocks,
     rfx::BoundTables<NUM_FEATS> *__restrict__ d_bound, const int *__restrict__ d_lookup_counts) {{
   __shared__ rfx::BindingStorage<NUM_FEATS> s_bind;
-  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch, d_lookup_counts}};
+  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch, d_lookup_counts, {"c_ext_feat" if tile_order is not None else "nullptr"}}};
   rfx::bind_once<NUM_FEATS, 1024, HAS_SPLIT>(s_bind, d_bound, io, tile_bytes, c_lookup_bytes, c_bag_bytes,
                                   c_cand_begin, c_cand_gran, d_schedule_choice, {fixed_arg},
                                   grid_blocks);
 }}
 ''' if bind_once else ''
 
-        outlier_kernel = '''
+        outlier_kernel = f'''
 // Finds the bags that are too long for their feature's schedule (one thread per bag).
 extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
     const int64_t *__restrict__ d_io_ptrs, const char *__restrict__ d_arg_buffers,
     const int64_t *__restrict__ d_arg_buffer_offsets, const int batch,
-    OutlierSpace *__restrict__ d_outliers) {
-  const rfx::IoView io{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch};
+    OutlierSpace *__restrict__ d_outliers) {{
+  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch, nullptr,
+                       {"c_ext_feat" if tile_order is not None else "nullptr"}}};
   rfx::find_outliers<NUM_FEATS>(d_outliers, io, c_long_thr, c_lookup_bytes);
-}
+}}
 ''' if outliers else ''
         outlier_begin = f'''
   // the parts of the outlier bags of this batch (0: none, or more than the list holds)
@@ -489,7 +523,7 @@ extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
       const int entry = d_outliers->partmap[tile];
       const rfx::OutlierEntry e = d_outliers->entries[entry];
       const int part = tile - e.first;
-      const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[e.feat]);
+      const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[io.ext_of(e.feat)]);
       const int *indices = io.indices(e.feat);
       const int *offsets = io.offsets(e.feat);
       const int embed_dim_offset = c_embed_dim_offsets[e.feat];
@@ -503,6 +537,50 @@ extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
   __syncthreads();
   if (threadIdx.x == 0) rfx::outliers_done(d_outliers);
 ''' if outliers else ''
+        if drawn_tail:
+            loop_head = f'''  // The last DRAWN_TAIL passes of the walk are drawn: tickets of this workgroup's XCD (of the
+  // whole device for a flat walk) count on from static_last.
+  rfx::TailTickets *const d_tickets = d_outliers;
+  __shared__ int s_ticket[2];
+  const int static_last = max(0, walk_last - DRAWN_TAIL * walk_step);
+  int walk = walk_first, ticket_slot = 0, next_ticket = 0;
+  bool drawing = false;
+  for (;;) {{
+    int at = 0;
+    if (!drawing) {{
+      if (walk < static_last) {{
+        at = walk;
+        walk += walk_step;
+      }} else {{
+        drawing = true;
+        if (threadIdx.x == 0) s_ticket[0] = rfx::draw_tail_ticket(d_tickets, xcd);
+        continue;
+      }}
+    }} else {{
+      __syncthreads();                         // the ticket is there, the previous tile is done
+      at = static_last + s_ticket[ticket_slot];
+      if (at >= walk_last) break;
+      // the next ticket: its value is needed only when this tile is done, so the round trip
+      // hides behind the tile
+      if (threadIdx.x == 0) next_ticket = rfx::draw_tail_ticket(d_tickets, xcd);
+      ticket_slot ^= 1;
+    }}
+    int tile = at;
+    if (by_xcd) {{
+      const int seg = at / seg_len;
+      tile = (seg * XCDS + xcd) * seg_len + (at - seg * seg_len);
+    }}
+    if (tile >= total_tiles) {{
+      if (drawing && threadIdx.x == 0) s_ticket[ticket_slot] = next_ticket;
+      continue;
+    }}
+'''
+            loop_tail = '''    if (drawing && threadIdx.x == 0) s_ticket[ticket_slot] = next_ticket;
+'''
+            outlier_end = '''
+  __syncthreads();
+  if (threadIdx.x == 0) rfx::tail_tickets_done(d_tickets);
+'''
         drain_func = f'''
 // Sums mid-size bags from the workgroup's list for as long as the calling wavefront gets one.
 __device__ __noinline__ void DrainMidBags(
@@ -511,7 +589,7 @@ __device__ __noinline__ void DrainMidBags(
   const int lane = threadIdx.x & 63;
   int feat = 0, bag = 0;
   while (rfx::mid_queue_pop(q, &feat, &bag)) {{
-    const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[feat]);
+    const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[io.ext_of(feat)]);
     const int *indices = io.indices(feat);
     const int *offsets = io.offsets(feat);
     const int beg = __builtin_amdgcn_readfirstlane(offsets[bag]);
@@ -531,7 +609,7 @@ __device__ __noinline__ void DrainMidBags(
     const int *indices = rfx::global_ptr<int>(rfx::uniform64(s_bind.indices_addr[feat_idx]));
     const int *offsets = rfx::global_ptr<int>(rfx::uniform64(s_bind.offsets_addr[feat_idx]));
     const int {vars_.one_per_bag} = __builtin_amdgcn_readfirstlane(s_bind.one_per_bag[feat_idx]);
-''' if keep_addrs else f'''    const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[feat_idx]);
+''' if keep_addrs else f'''    const char *table = rfx::global_ptr<char>(d_embed_table_ptrs[io.ext_of(feat_idx)]);
     const int *indices = io.indices(feat_idx);
     const int *offsets = io.offsets(feat_idx);
     const int {vars_.one_per_bag} = 0;
@@ -551,7 +629,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
 {bind_decl}
   __shared__ KnlTempStorage s;
 {stage_decl}{timing_init}
-  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch, d_lookup_counts}};
+  const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch, d_lookup_counts, {"c_ext_feat" if tile_order is not None else "nullptr"}}};
 {bind_call}
 {timing_bound}
 {outlier_begin}
@@ -623,7 +701,7 @@ static int launch_kernels(const recom_process_args *a, void *workspace) {
   const char *arg_buffers = static_cast<const char *>(a->d_arg_buffers);
   int batch = a->batch, tile_arg = tile_bytes, xcd_arg = xcd_segments;
   int stride_arg = static_cast<int>(row_stride);
-  void *outlier_space = OUTLIERS ? static_cast<char *>(workspace) + SPLIT_BYTES : nullptr;
+  void *outlier_space = OUTLIERS || DRAWN_TAIL > 0 ? static_cast<char *>(workspace) + SPLIT_BYTES : nullptr;
   void *bound = BIND_ONCE ? static_cast<char *>(workspace) + BOUND_OFFSET : nullptr;
   // The caller's events take the begin of the call's first kernel and the end of its last
   // (the fused kernel): a library that launches a kernel ahead of the fused one is timed whole.
@@ -705,7 +783,7 @@ extern "C" __global__ void __launch_bounds__(256) ScratchClearKnl(char *__restri
 #if RFX_HAS_SPLIT
   for (int f = blockIdx.y; f < NUM_FEATS; f += gridDim.y) {
     if (c_split_region[f] < 0) continue;
-    const int dim = c_embed_dim_offsets[f + 1] - c_embed_dim_offsets[f];
+    const int dim = c_embed_dims[f];
     int *counters = reinterpret_cast<int *>(ws) + c_split_region[f] +
                     static_cast<long long>(rfx::kSplitMaxTiles) * dim;
     for (int i = first; i < rfx::kSplitMaxTiles; i += step) counters[i] = 0;
@@ -717,6 +795,12 @@ extern "C" __global__ void __launch_bounds__(256) ScratchClearKnl(char *__restri
     int *hdr = reinterpret_cast<int *>(&sp->hdr);
     for (int i = first; i < static_cast<int>(sizeof(rfx::OutlierHeader) / 4); i += step) hdr[i] = 0;
     for (int i = first; i < OutlierSpace::kCap; i += step) sp->counters[i] = 0;
+  }
+#endif
+#if RFX_DRAWN_TAIL
+  if (blockIdx.y == 0) {
+    int *tickets = reinterpret_cast<int *>(ws + SPLIT_BYTES);
+    for (int i = first; i < static_cast<int>(sizeof(rfx::TailTickets) / 4); i += step) tickets[i] = 0;
   }
 #endif
   (void)ws; (void)first; (void)step;
@@ -865,7 +949,8 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
              tune: bool = False, timing: bool = False, timing_branch: bool = False,
              fixed_task_block_nums: List[int] = None, tile_bytes: int = None,
              xcd_aware: bool = False, lookup_overhead_bytes: int = None,
-             xcd_segments: int = 8, outliers: bool = False, bind_once: bool = None) -> None:
+             xcd_segments: int = 8, outliers: bool = False, bind_once: bool = None,
+             tile_order: List[int] = None, drawn_tail: int = 0) -> None:
         """Write the device source.  ``occupancy`` = workgroups per CU the kernel is built and
         launched for (``__launch_bounds__`` budget, persistent grid size, and a dynamic-LDS pad
         that keeps further workgroups off the CU); ``tune`` is accepted for signature
@@ -879,7 +964,8 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
                                  fixed_task_block_nums=fixed_task_block_nums,
                                  tile_bytes=tile_bytes, xcd_aware=xcd_aware,
                                  lookup_overhead_bytes=lookup_overhead_bytes,
-                                 xcd_segments=xcd_segments, outliers=outliers, bind_once=bind_once)
+                                 xcd_segments=xcd_segments, outliers=outliers, bind_once=bind_once,
+                                 tile_order=tile_order, drawn_tail=drawn_tail)
         code += self.emit_process_func(timing=timing, occupancy=occupancy)
         code += self.emit_get_concurrent_blocks_func(occupancy=occupancy)
         code += self.emit_process_ops()

@@ -41,12 +41,21 @@ struct IoView {
   // optional: the lookups of every feature in this batch as the caller knows them (a hint for
   // the binding, which otherwise reads offsets[batch] of every feature)
   const int *__restrict__ counts = nullptr;
+  // optional: the caller's number of every feature of the kernel.  A kernel emitted with a tile
+  // order lays the features out in its tile space in an order of its own and numbers them by
+  // their place there; whatever the caller passes per feature -- addresses, counts, tables -- is
+  // found through this table (null: the kernel's numbers are the caller's).
+  const int *__restrict__ ext = nullptr;
 
+  __device__ __forceinline__ int ext_of(int f) const { return ext ? ext[f] : f; }
+  __device__ __forceinline__ int count(int f) const { return counts[ext_of(f)]; }
   __device__ __forceinline__ int64_t offsets_addr(int f) const {
+    f = ext_of(f);
     if (io_ptrs) return io_ptrs[2 * f + 1];
     return reinterpret_cast<int64_t>(arg_base) + arg_offsets[f];
   }
   __device__ __forceinline__ int64_t indices_addr(int f) const {
+    f = ext_of(f);
     if (io_ptrs) return io_ptrs[2 * f];
     return reinterpret_cast<int64_t>(arg_base) + arg_offsets[f] +
            alignmem((static_cast<int64_t>(batch) + 1) * 4);
@@ -55,6 +64,7 @@ struct IoView {
   // inputs have (no branch: the binding issues these loads for all features at once).
   __device__ __forceinline__ void addrs(int f, int64_t &indices_at, int64_t &offsets_at) const {
     typedef long long pair_t __attribute__((ext_vector_type(2), aligned(8)));
+    f = ext_of(f);
     const bool ptrs = io_ptrs != nullptr;
     // pointer table: {indices, offsets} of f; packed form: {byte offset of f, of f + 1}
     const int64_t *src = ptrs ? io_ptrs + 2 * f : arg_offsets + f;
@@ -241,7 +251,7 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     io.addrs(f, idx_at[k], offs_at[k]);
     table_at[k] = 0;
     // (the once-per-launch binding kernel has no use for the tables' addresses and passes none)
-    if constexpr (BindingStorage<F>::kKeepAddrs) table_at[k] = table_ptrs ? table_ptrs[f] : 0;
+    if constexpr (BindingStorage<F>::kKeepAddrs) table_at[k] = table_ptrs ? table_ptrs[io.ext_of(f)] : 0;
     cand[k] = f;
     if constexpr (!ONE_CAND) {
       const int first = cand_begin[f];
@@ -265,7 +275,7 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
       int first_lookup = 0;
       int64_t lookups;
       if (io.counts) {                        // one array for all features instead of a line each
-        lookups = io.counts[f];
+        lookups = io.count(f);
       } else {
         const int *offs = global_ptr<int>(offs_at[k]);
         first_lookup = offs[0];

@@ -118,4 +118,34 @@ template <typename Space> __device__ __forceinline__ void outliers_done(Space *s
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The drawn end of the tile walk (emit option drawn_tail = N): the last N passes of a workgroup
+// over the tile space are not dealt out by the stride; the workgroups of an XCD draw them from a
+// ticket counter of that XCD (one cache line each), so that a workgroup whose tiles were cheap
+// takes over from one whose tiles were dear.  It pays together with a tile order that puts the
+// cheap tiles last (a model of a thousand small features, five tiles per workgroup: 70.2 ->
+// 67.8 us; alone, or on a model of 100 features with ten tiles per workgroup, nothing).  One
+// thread draws, the next ticket is requested before the current tile runs, the workgroup agrees
+// through LDS; the last workgroup to finish puts the counters back to zero.
+// ---------------------------------------------------------------------------------------------
+struct TailTickets {
+  int next[8][32];                           // per XCD, each on a cache line of its own
+  int finished;                              // workgroups that are done
+  int pad[31];
+};
+
+__device__ __forceinline__ int draw_tail_ticket(TailTickets *t, const int xcd) {
+  return __hip_atomic_fetch_add(&t->next[xcd][0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// by one thread of every workgroup when it has drawn its last ticket
+__device__ __forceinline__ void tail_tickets_done(TailTickets *t) {
+  const int done = __hip_atomic_fetch_add(&t->finished, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (done == static_cast<int>(gridDim.x) - 1) {
+    for (int x = 0; x < 8; ++x)
+      __hip_atomic_store(&t->next[x][0], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&t->finished, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 } // namespace rfx

@@ -25,7 +25,8 @@ def emit_model(output_dir: str, feat_schedules: FeatSchedules, occupancy: Option
                fixed_task_block_nums: List[int] = None, tile_bytes: int = None,
                debug: bool = False, host: bool = True, xcd_aware: bool = True,
                lookup_overhead_bytes: int = None, xcd_segments: int = DEFAULT_XCD_SEGMENTS,
-               outliers: bool = False, bind_once: bool = None) -> None:
+               outliers: bool = False, bind_once: bool = None, tile_order: List[int] = None,
+               drawn_tail: int = 0) -> None:
     os.makedirs(output_dir, exist_ok=True)
     emitter = CodeEmitter(feat_schedules)
     if host:
@@ -33,7 +34,7 @@ def emit_model(output_dir: str, feat_schedules: FeatSchedules, occupancy: Option
     emitter.emit(f"{output_dir}/process.hip", occupancy=occupancy, timing=timing, inline=inline,
                  tune=tune, fixed_task_block_nums=fixed_task_block_nums, tile_bytes=tile_bytes,
                  xcd_aware=xcd_aware, lookup_overhead_bytes=lookup_overhead_bytes, xcd_segments=xcd_segments,
-                 outliers=outliers, bind_once=bind_once)
+                 outliers=outliers, bind_once=bind_once, tile_order=tile_order, drawn_tail=drawn_tail)
     emitter.emit_cmake_list(f"{output_dir}/CMakeLists.txt", code_fname="process.hip",
                             host_fname="preprocess.cpp" if host else None, debug=debug)
     emitter.dump_key(f"{output_dir}/schedule.json")

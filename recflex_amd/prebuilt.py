@@ -113,6 +113,10 @@ def _tuned(wl: Workload, fname: str) -> ModelSpec:
         kwargs.update(xcd_aware=True, xcd_segments=doc["xcd_segments"])
     else:
         kwargs.update(xcd_aware=False)      # the tuned walk is the flat one
+    if isinstance(doc, dict) and doc.get("tile_order"):
+        kwargs["tile_order"] = [int(f) for f in doc["tile_order"]]
+    if isinstance(doc, dict) and doc.get("drawn_tail"):
+        kwargs["drawn_tail"] = int(doc["drawn_tail"])
     if isinstance(doc, dict) and doc.get("outliers"):
         kwargs["outliers"] = True
     return ModelSpec(wl, fs, occupancy, kwargs)
@@ -289,6 +293,24 @@ def _wide(num_features: int = 1500, name: str = "wide") -> ModelSpec:
     return _default(wl)
 
 
+def _ordered(spec: ModelSpec, name: str, seed: int, drawn_tail: int = 0, **emit_kwargs) -> ModelSpec:
+    """The same model and schedules with the features laid out in the kernel's tile space in a
+    random order (``tile_order``) and, if asked for, the last passes of the tile walk drawn."""
+    order = [int(f) for f in np.random.default_rng(seed).permutation(len(spec.feat_schedules))]
+    kwargs = dict(spec.emit_kwargs, tile_order=order, **emit_kwargs)
+    if drawn_tail:
+        kwargs["drawn_tail"] = drawn_tail
+    return spec._replace(workload=spec.workload._replace(name=name), emit_kwargs=kwargs)
+
+
+def _c3s_ordered() -> ModelSpec:
+    """c3s_outliers' model (integer tables, every tenth feature split) without outlier tiles, in
+    a random tile order with the last two passes drawn."""
+    spec = _c3s_outliers()
+    spec = spec._replace(emit_kwargs={k: v for k, v in spec.emit_kwargs.items() if k != "outliers"})
+    return _ordered(spec, "c3s_ordered", 11, drawn_tail=2)
+
+
 _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c1": lambda: _default(make_workload("C1")),
     "c2": lambda: _default(make_workload("C2")),
@@ -316,6 +338,13 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     # by the binding kernel all the same (an emit option)
     "c3s_bind_once": lambda: _default(make_workload("C3", batch=192, max_rows=60_000), bind_once=True),
     "c3s_outliers": _c3s_outliers,
+    # tile orders: features in a random order in the tile space (addresses kept in LDS / read per
+    # tile / bound once per launch; with split regions, with outlier tiles), drawn ends
+    "c3s_ordered": _c3s_ordered,
+    "c3s_outliers_ordered": lambda: _ordered(_c3s_outliers(), "c3s_outliers_ordered", 12),
+    "wide_ordered": lambda: _ordered(_wide(), "wide_ordered", 13, drawn_tail=1),
+    "wider_ordered": lambda: _ordered(_wide(2500, "wider"), "wider_ordered", 14, drawn_tail=3),
+    "onehots_ordered": lambda: _ordered(_onehots(), "onehots_ordered", 15, drawn_tail=8),
     # fp16 and int8 tables with outlier tiles (integer-valued: sums exact)
     "c4s_outliers": lambda: _default(make_workload("C4", batch=128, num_features=48, max_rows=30_000)
                                      ._replace(name="c4s_outliers", table_values="integer"), outliers=True),

@@ -395,6 +395,39 @@ def measure_kernel_events(librecom_path: str, table_shapes: Sequence[Tuple[int, 
         return None
 
 
+def measure_feature_ticks(librecom_path: str, table_shapes: Sequence[Tuple[int, int]],
+                          data_types: Sequence[str], data_npzs: Sequence[str], output_path: str,
+                          tile_bytes: int = 0, xcd_segments: int = 0, repeats: int = 3,
+                          gpu_id: int = None) -> Optional[np.ndarray]:
+    """Workgroup ticks per feature of a timing build of the whole model, summed over the
+    batches (mean of ``repeats`` launches each); one number per line of ``output_path``."""
+    try:
+        _pin_gpu(gpu_id)
+        import torch
+        from recflex_amd.rec_modules import FeatEmbed
+
+        dev = torch.device("cuda", torch.cuda.current_device())
+        tables = [make_table(s, t, dev, ones=False) for s, t in zip(table_shapes, data_types)]
+        layer = FeatEmbed(dev, embed_tables=tables, librecom=librecom_path)
+        per_feat = [load_batches(p) for p in data_npzs]
+        total = np.zeros(len(per_feat), dtype=np.float64)
+        for k in range(len(per_feat[0])):
+            bound = layer.bind_inputs([torch.from_numpy(b[k][0]).to(dev) for b in per_feat],
+                                      [torch.from_numpy(b[k][1]).to(dev) for b in per_feat])
+            out = layer.forward_indices(bound, tile_bytes=tile_bytes, xcd_segments=xcd_segments)
+            acc = np.zeros(len(per_feat), dtype=np.float64)
+            for _ in range(repeats):
+                _, ticks = layer.forward_indices(bound, timing=True, out=out, tile_bytes=tile_bytes,
+                                                 xcd_segments=xcd_segments)
+                acc += ticks.numpy()
+            total += acc / repeats
+        _write_atomically(output_path, "".join(f"{v:.1f}\n" for v in total))
+        return total
+    except Exception as e:
+        print(f"[{librecom_path}] Exception {type(e).__name__}: {e}", flush=True)
+        return None
+
+
 class KernelTimer:
     """Times the FusedKnl of several libraries of one model over the same tables and batches,
     which stay on the device between calls (the production-build climb times hundreds of

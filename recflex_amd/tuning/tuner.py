@@ -40,7 +40,8 @@ from recflex_amd.task_manager import TaskManager
 from recflex_amd.parser import (parse_raw_data_batches, parse_table_shapes, parse_table_dtypes,
                                 parse_schedule_types, parse_knl_total_time, parse_knl_batch_times)
 
-from .measure import (measure_single_feat, rocprof_profile, measure_task_blocks,
+from .measure import (measure_single_feat, rocprof_profile, measure_task_blocks, measure_feature_ticks,
+                      tiles_per_feature,
                       measure_naive_candidate, measure_kernel_events, measure_tournament,
                       save_batches, KernelTimer, PROFILE_PASSES, PROFILE_WARMUP_PASSES)
 
@@ -81,6 +82,14 @@ class TuneConfig(NamedTuple):
     outliers: Optional[bool] = None
     # undecided (None): kept only if the whole call is faster by this share on the samples
     outliers_min_gain: float = 0.02
+    # the order of the features in the kernel's tile space and a drawn end of the tile walk
+    # (Tuner.decide_walk): True / False, or None = tried for models of at least
+    # ``walk_stage_min_feats`` features whose workgroups get fewer than
+    # ``walk_stage_max_tiles`` tiles each on the samples (with more, the deal evens out by itself)
+    walk_stage: Optional[bool] = None
+    walk_stage_min_feats: int = 256
+    walk_stage_max_tiles: float = 8.0
+    walk_min_gain: float = 0.01
     # local-stage interference: "model" = every candidate of every feature is compiled into one
     # kernel of the whole model and timed while all other features run beside it;
     # "replicate" = per feature, the candidates side by side over the same data, replicated
@@ -301,14 +310,15 @@ class Tuner:
                    occupancy: int, inline: bool = True, timing: bool = False, tune: bool = False,
                    fixed_task_block_nums: List[int] = None, debug: bool = False,
                    tile_bytes: int = None, host: bool = True, xcd_segments: int = 0,
-                   outliers: bool = False) -> None:
+                   outliers: bool = False, tile_order: List[int] = None, drawn_tail: int = 0) -> None:
         os.makedirs(output_dir, exist_ok=True)
         emitter = CodeEmitter(feat_schedules)
         if host:
             emitter.emit_host(f"{output_dir}/preprocess.cpp", fixed_task_block_nums=fixed_task_block_nums)
         emitter.emit(f"{output_dir}/process.hip", occupancy=occupancy, timing=timing, inline=inline, tune=tune,
                      fixed_task_block_nums=fixed_task_block_nums, tile_bytes=tile_bytes,
-                     xcd_aware=xcd_segments > 0, xcd_segments=max(xcd_segments, 1), outliers=outliers)
+                     xcd_aware=xcd_segments > 0, xcd_segments=max(xcd_segments, 1), outliers=outliers,
+                     tile_order=tile_order, drawn_tail=drawn_tail)
         emitter.emit_cmake_list(f"{output_dir}/CMakeLists.txt", code_fname="process.hip",
                                 host_fname="preprocess.cpp" if host else None,
                                 subdirs=self.basic.subdirs, includes=self.basic.includes, links=self.basic.links,
@@ -981,6 +991,114 @@ class Tuner:
               f"{t_on:.0f} ns with, {t_off:.0f} ns without)", flush=True)
         return keep
 
+    def sample_tiles(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
+                     tile_bytes: int, tune_config: TuneConfig) -> np.ndarray:
+        """Tiles the binding gives every feature of this mix, summed over the sampled batches."""
+        metas = [s.meta for s, _ in sched_params]
+        tiles = np.zeros(self.num_feats)
+        batches = getattr(self, "batches", None) or []
+        for k in range(len(batches[0]) if batches else 0):
+            tiles += tiles_per_feature([feat[k][1] for feat in batches],
+                                       [m.row_bytes + INDEX_BYTES for m in metas],
+                                       [m.embed_dim * 4 + BAG_FIXED_BYTES for m in metas],
+                                       [s.TileGranularity(p) for s, p in sched_params],
+                                       tile_bytes or tune_config.tile_bytes,
+                                       grid_blocks=tune_config.sm_count * occupancy)
+        return tiles
+
+    def tile_time_order(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
+                        tile_bytes: int, xcd_segments: int, tune_config: TuneConfig
+                        ) -> Optional[List[int]]:
+        """The features by the time one of their tiles takes, dearest first: a timing build of
+        the mix as it ships (tick counters per feature) is run on the samples, and every
+        feature's ticks are divided by the tiles the binding gives it.  (The tournament's tile
+        times do not serve: its kernel holds every candidate, and an order by its figures was no
+        better than the model's own.)  None if nothing can be told apart."""
+        output_dir = f"{self.basic.codegen_dir}/walk_timing/o{occupancy}"
+        self.emit_codes(output_dir=output_dir, feat_schedules=sched_params, occupancy=occupancy,
+                        inline=tune_config.inline, timing=True, debug=tune_config.debug,
+                        tile_bytes=tile_bytes, xcd_segments=max(xcd_segments, 0))
+        self._schedule_builds([(output_dir, f"{output_dir}/build")], tune_config)
+        result = f"{output_dir}/feature_ticks.txt"
+        if os.path.exists(result):
+            os.remove(result)
+        manager = None if tune_config.in_process else TaskManager(tune_config.gpu_ids[0:1])
+        if manager:
+            release_device_memory()
+        args = (f"{output_dir}/build/librecom.so", self.table_shapes, self.data_types, self.data_npzs,
+                result, tile_bytes, xcd_segments)
+        self._run_measure(manager, tune_config, measure_feature_ticks, args)
+        if manager:
+            manager.join()
+        if not os.path.exists(result):
+            return None
+        with open(result) as f:
+            ticks = [float(line) for line in f if line.strip()]
+        tiles = self.sample_tiles(sched_params, occupancy, tile_bytes, tune_config)
+        if len(ticks) != self.num_feats:
+            return None
+        # features of one kind (schedule, parameters, row type and width) share one figure: a
+        # single feature's few tiles are too few to tell its time from its neighbours'
+        kinds: Dict[tuple, List[float]] = {}
+        kind_of = [(type(s).__name__, tuple(p), s.meta.data_type, s.meta.embed_dim) for s, p in sched_params]
+        for k, t, n in zip(kind_of, ticks, tiles):
+            acc = kinds.setdefault(k, [0.0, 0.0])
+            acc[0] += t
+            acc[1] += n
+        per_tile = [kinds[k][0] / kinds[k][1] if kinds[k][1] > 0 else 0.0 for k in kind_of]
+        if len(set(round(v) for v in per_tile)) < 3:
+            return None
+        return sorted(range(self.num_feats), key=lambda f: (-per_tile[f], f))
+
+    def decide_walk(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
+                    measured_times: Dict[int, Dict[int, List[float]]], tile_bytes: int,
+                    xcd_segments: int, outliers: bool, tune_config: TuneConfig
+                    ) -> Tuple[Optional[List[int]], int]:
+        """(tile_order, drawn_tail) for ``optimal/``, by measurement.  With the features sorted
+        by their time per tile, the strided deal hands every workgroup one tile of each kind,
+        and a drawn end then has cheap tiles to fill it with: worth 5 and 9 % on a model of a
+        thousand small features whose workgroups get five tiles each, nothing on one of a
+        hundred features and ten tiles per workgroup.  The mix is built as it is, ordered, and
+        ordered with the last two passes drawn, all three are timed on the samples like
+        contenders of the global stage, and a variant is kept if it gains
+        ``TuneConfig.walk_min_gain``."""
+        want = tune_config.walk_stage
+        if want is None and self.num_feats >= tune_config.walk_stage_min_feats:
+            batches = getattr(self, "batches", None) or [[]]
+            per_workgroup = (self.sample_tiles(sched_params, occupancy, tile_bytes, tune_config).sum()
+                             / max(1, len(batches[0])) / (tune_config.sm_count * occupancy))
+            want = per_workgroup < tune_config.walk_stage_max_tiles
+        order = (self.tile_time_order(sched_params, occupancy, tile_bytes, xcd_segments, tune_config)
+                 if want else None)
+        if order is None:
+            return None, 0
+        variants = {"as_is": (None, 0), "ordered": (order, 0)}
+        if not outliers:
+            variants["ordered_drawn"] = (order, 2)
+        dirs = {name: f"{self.basic.codegen_dir}/walk_{name}/o{occupancy}" for name in variants}
+        jobs = []
+        for name, (tile_order, drawn_tail) in variants.items():
+            self.emit_codes(output_dir=dirs[name], feat_schedules=sched_params, occupancy=occupancy,
+                            inline=tune_config.inline, debug=tune_config.debug, tile_bytes=tile_bytes,
+                            xcd_segments=max(xcd_segments, 0), outliers=outliers,
+                            tile_order=tile_order, drawn_tail=drawn_tail)
+            jobs.append((dirs[name], f"{dirs[name]}/build"))
+        self._schedule_builds(jobs, tune_config)
+        manager = self._measure_manager(tune_config)
+        if tune_config.profiler == "rocprofv3" or manager:
+            release_device_memory()
+        cfg = tune_config._replace(remeasure=True)
+        for output_dir in dirs.values():
+            self._kernel_time(output_dir, cfg, manager)
+        if manager:
+            manager.join()
+        times = {name: self._read_kernel_time(dirs[name], tune_config) for name in variants}
+        best = min(times, key=times.get)
+        keep = best if times[best] < times["as_is"] * (1.0 - tune_config.walk_min_gain) else "as_is"
+        print("tile walk: " + ", ".join(f"{name} {t:.0f} ns" for name, t in times.items())
+              + f": {keep.replace('_', ' ')}", flush=True)
+        return variants[keep]
+
     def solve(self, measured_times: Dict[int, Dict[int, List[float]]],
               tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
         occu_opt_sched_params = self.select_per_occupancy(measured_times, tune_config.occupancies)
@@ -1003,20 +1121,25 @@ class Tuner:
         if outliers is None:
             outliers = self.decide_outliers(opt_sched_params, opt_occupancy, tile_bytes, xcd_segments,
                                             tune_config)
+        tile_order, drawn_tail = self.decide_walk(opt_sched_params, opt_occupancy, measured_times,
+                                                  tile_bytes, xcd_segments, bool(outliers), tune_config)
         # a contender whose library came out of the compile cache (the same source had been built
         # in another directory) has no host module of its own: optimal/ is then built in place
         import glob
         host_missing = not glob.glob(f"{optimal}/build/recom_host*.so")
-        if climbed or tile_bytes != tune_config.tile_bytes or xcd_segments or outliers or host_missing:
+        if climbed or tile_bytes != tune_config.tile_bytes or xcd_segments or outliers or host_missing \
+                or tile_order is not None or drawn_tail:
             # make the winning launch parameters the defaults of the optimal library
             self.emit_codes(output_dir=optimal, feat_schedules=opt_sched_params, occupancy=opt_occupancy,
                             inline=tune_config.inline, debug=tune_config.debug, tile_bytes=tile_bytes,
-                            xcd_segments=max(xcd_segments, 0), outliers=outliers)
+                            xcd_segments=max(xcd_segments, 0), outliers=outliers,
+                            tile_order=tile_order, drawn_tail=drawn_tail)
             shutil.rmtree(f"{optimal}/build", ignore_errors=True)   # the copied CMake cache names another dir
             compile_build(f"{optimal}/build")
         with open(f"{optimal}/schedule.json", "w") as f:
             json.dump({"occupancy": opt_occupancy, "tile_bytes": tile_bytes,
                        "xcd_segments": max(xcd_segments, 0), "outliers": bool(outliers),
+                       "tile_order": tile_order, "drawn_tail": int(drawn_tail),
                        "schedules": CodeEmitter(opt_sched_params).serialize_config()}, f, indent=1)
         return opt_occupancy, opt_sched_params
 

@@ -242,6 +242,57 @@ def test_outlier_tiles_are_emitted_on_request():
         em.emit_kernel(occupancy=4, outliers=True, timing=True)
 
 
+def _table(src: str, name: str):
+    import re
+    body = re.search(r"\b" + name + r"\[\] = \{(.*?)\};", src, re.S).group(1)
+    return [int(v) for v in body.replace("\n", " ").split(",") if v.strip()]
+
+
+def test_tile_order_permutes_the_kernels_tables_and_nothing_the_host_sees():
+    """tile_order: inside the kernel a feature's number is its place in the tile space -- every
+    per-feature table is emitted in that order, the output columns stay where the model has
+    them, and what the caller passes per feature is found through c_ext_feat.  The identity and
+    no order at all emit the same source; the host-side description of the library does not
+    move."""
+    fs = [default_schedule(MetaData(32), 4), default_schedule(MetaData(128), 1),
+          default_schedule(MetaData(8), 30), default_schedule(MetaData(64, "half"), 900)]
+    em = CodeEmitter(fs)
+    plain = em.emit_kernel(occupancy=4)
+    assert em.emit_kernel(occupancy=4, tile_order=[0, 1, 2, 3]) == plain
+    assert "c_ext_feat" not in plain and "#define RFX_TILE_ORDER 0" in plain
+    order = [2, 0, 3, 1]
+    src = em.emit_kernel(occupancy=4, tile_order=order)
+    assert "#define RFX_TILE_ORDER 1" in src and _table(src, "c_ext_feat") == order
+    for name in ("c_cand_func_ids", "c_cand_gran", "c_embed_dims", "c_lookup_bytes", "c_bag_bytes"):
+        assert _table(src, name) == [_table(plain, name)[f] for f in order], name
+    offs = _table(plain, "c_embed_dim_offsets")
+    assert offs == [0, 32, 160, 168, 232]
+    assert _table(src, "c_embed_dim_offsets") == [offs[f] for f in order] + [232]
+    assert _table(src, "c_split_region") == [_table(plain, "c_split_region")[f] for f in order]
+    assert "d_lookup_counts, c_ext_feat}" in src and "d_lookup_counts, nullptr}" in plain
+    assert em.emit_process_func(occupancy=4) == CodeEmitter(fs).emit_process_func(occupancy=4)
+    with pytest.raises(AssertionError):
+        em.emit_kernel(occupancy=4, tile_order=[0, 1, 2, 2])
+    with pytest.raises(AssertionError):
+        em.emit_kernel(occupancy=4, tile_order=order, timing=True)
+
+
+def test_drawn_tail_takes_its_ticket_counters_from_the_workspace():
+    """drawn_tail=N: the last N passes of the tile walk are drawn; the ticket counters live in
+    the workspace where an outlier list would (never both), and the kernel that clears a static
+    workspace clears them."""
+    fs = [default_schedule(MetaData(32), 4), default_schedule(MetaData(128), 1)]
+    em = CodeEmitter(fs)
+    src = em.emit_kernel(occupancy=4, drawn_tail=2) + em.emit_process_func(occupancy=4)
+    assert "#define RFX_DRAWN_TAIL 2" in src and "using OutlierSpace = rfx::TailTickets;" in src
+    assert "rfx::draw_tail_ticket(d_tickets, xcd)" in src and "rfx::tail_tickets_done(d_tickets)" in src
+    assert "sizeof(rfx::TailTickets) / 4" in src
+    plain = em.emit_kernel(occupancy=4)
+    assert "#define RFX_DRAWN_TAIL 0" in plain and "draw_tail_ticket" not in plain
+    with pytest.raises(AssertionError):
+        em.emit_kernel(occupancy=4, drawn_tail=2, outliers=True)
+
+
 def test_launch_bounds_carry_wavefronts_per_simd_not_workgroups_per_cu():
     """hipcc reads the second argument of __launch_bounds__ as wavefronts per SIMD: a build of
     64-thread workgroups at 20 per CU has to ask for 5, one of 128-thread workgroups at 6 for 3."""

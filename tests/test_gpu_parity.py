@@ -306,6 +306,52 @@ def test_lookup_count_hint_sizes_tiles_and_nothing_else(name):
         assert bad.size == 0, f"{label}: {len(bad)} elements differ, first at {bad[:5].tolist()}"
 
 
+@pytest.mark.parametrize("name", ["c3s_ordered", "c3s_outliers_ordered", "wide_ordered", "wider_ordered",
+                                  "onehots_ordered"])
+def test_tile_order_and_drawn_end_change_no_bit(name):
+    """A library emitted with ``tile_order`` numbers the features inside the kernel by their
+    place in the tile space and finds what the caller passes per feature through a table; with
+    ``drawn_tail`` the last passes of the walk are drawn from ticket counters.  Neither may
+    change a bit of the output: random orders on a model that keeps its addresses in LDS (with
+    split regions; with outlier tiles), one that reads them per tile, one bound once per launch,
+    and the row-copy template with every tile drawn.  Three launches on one workspace (the
+    ticket counters must be back at zero), with and without the lookup-count hint, also through
+    the entry point that uses the library's static workspace.  Integer-valued tables: bit for
+    bit against the oracle."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.workloads import gen_inputs, gen_tables
+
+    spec = prebuilt.model_spec(name)
+    wl = spec.workload
+    assert wl.table_values == "integer" and spec.emit_kwargs.get("tile_order")
+    dev = torch.device("cuda", 0)
+    print(f"[case] {name}: F={wl.num_features} B={wl.batch} {sorted(k for k in spec.emit_kwargs)}", flush=True)
+    tables = gen_tables(wl, dev)
+    host_tables = [t.cpu().numpy() for t in tables]
+    layer = FeatEmbed(dev, embed_tables=tables, librecom=require_lib(name))
+    for launch in range(3):
+        indices, offsets = gen_inputs(wl._replace(seed=wl.seed + 31 * launch))
+        bound = layer.bind_inputs([torch.from_numpy(i).to(dev) for i in indices],
+                                  [torch.from_numpy(o).to(dev) for o in offsets])
+        if launch == 1:
+            bound = bound._replace(lookup_counts=None)
+        got = layer.forward_indices(bound).cpu().numpy()
+        want = oracle_output(wl, host_tables, indices, offsets)
+        bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+        assert bad.size == 0, f"launch {launch}: {len(bad)} elements differ, first at {bad[:5].tolist()}"
+    if layer.lib.info.static_workspace and layer.lib.workspace_bytes:
+        out = torch.full((wl.batch * wl.embed_dim_sum,), float("nan"), device=dev)
+        for _ in range(2):
+            layer.lib.process(layer.embed_table_ptrs.data_ptr(), out.data_ptr(), wl.batch,
+                              io_ptrs=bound.io_ptrs.data_ptr(), static_workspace=True,
+                              stream=torch.cuda.current_stream(dev).cuda_stream)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().reshape(want.shape)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 def test_gather_probe_runs():
     """The measurement aid of bench.py: fetches the rows of a batch and nothing else.  It must
     run to completion on ragged inputs (empty features, rows of 1 to 64 vectors) and take time."""

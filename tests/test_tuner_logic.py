@@ -389,6 +389,87 @@ def test_outlier_tiles_are_kept_only_if_the_call_is_faster(tmp_path, monkeypatch
     assert tuner.decide_outliers(mix, 4, 65536, 16, cfg) is False
 
 
+def test_tile_walk_is_decided_by_measurement(tmp_path, monkeypatch):
+    """The walk stage orders the features by the local stage's time per tile (dearest first),
+    builds the mix as it is, ordered, and ordered with a drawn end, and keeps the fastest only if
+    it gains ``walk_min_gain``; with outlier tiles no drawn end is tried; small models skip the
+    stage unless told otherwise."""
+    tuner = _tiny_tuner(tmp_path)
+    mix = [c[0] for c in tuner.feat_sched_param_candidates]
+    measured = {}
+    built, times = [], {}
+    monkeypatch.setattr(Tuner, "_schedule_builds", lambda self, jobs, cfg: built.extend(j[0] for j in jobs))
+    monkeypatch.setattr(Tuner, "_kernel_time", lambda self, d, cfg, mgr, tb=0, xs=0: None)
+    monkeypatch.setattr(Tuner, "_read_kernel_time",
+                        lambda self, d, cfg, tb=0, xs=0: times[d.split("/walk_")[1].split("/")[0]])
+    monkeypatch.setattr(Tuner, "tile_time_order", lambda self, sp, occ, tb, xs, cfg: [1, 0])
+    cfg = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=1, in_process=True,
+                     cluster_stage=False)
+    assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, cfg) == (None, 0) and not built
+    cfg = cfg._replace(walk_stage=True)
+    times.update(as_is=1000.0, ordered=940.0, ordered_drawn=900.0)
+    assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, cfg) == ([1, 0], 2)
+    assert len(built) == 3
+    drawn = open([d for d in built if "ordered_drawn" in d][0] + "/process.hip").read()
+    assert "#define RFX_DRAWN_TAIL 2" in drawn and "c_ext_feat" in drawn
+    times.update(as_is=1000.0, ordered=940.0, ordered_drawn=960.0)
+    assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, cfg) == ([1, 0], 0)
+    times.update(as_is=1000.0, ordered=995.0, ordered_drawn=996.0)      # within the margin
+    assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, cfg) == (None, 0)
+    del built[:]
+    times.update(as_is=1000.0, ordered=900.0)
+    assert tuner.decide_walk(mix, 4, measured, 65536, 16, True, cfg) == ([1, 0], 0)
+    assert len(built) == 2 and not any("drawn" in d for d in built)
+    # undecided: wide enough models whose workgroups get few tiles each
+    auto = cfg._replace(walk_stage=None, walk_stage_min_feats=2)
+    del built[:]
+    assert tuner.decide_walk(mix, 4, measured, 65536, 16, True, auto._replace(walk_stage_max_tiles=0.01)) == (None, 0)
+    assert not built
+    assert tuner.decide_walk(mix, 4, measured, 65536, 16, True, auto._replace(walk_stage_max_tiles=1e9)) == ([1, 0], 0)
+    assert tuner.decide_walk(mix, 4, measured, 65536, 16, True, auto._replace(walk_stage_min_feats=3)) == (None, 0)
+
+
+def test_tile_order_comes_from_the_ticks_of_the_mix_as_it_ships(tmp_path, monkeypatch):
+    """The order key is ticks per tile of a timing build of the chosen mix, pooled over the
+    features of one kind (schedule, parameters, row type, width): dearest kind first, features
+    of a kind in their own order; fewer than three distinct figures order nothing."""
+    import recflex_amd.tuning.tuner as tuner_mod
+    rng = np.random.default_rng(9)
+    dims, data = [16, 16, 64, 64, 32], []
+    for f in range(5):
+        lens = rng.integers(1, 6, 64)
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        data.append([(rng.integers(0, 100, off[-1]).astype(np.int32), off)])
+    cfg = BasicConfig("", [], "", "", str(tmp_path / "out"), block_threads=256, sample_batch_nums=1)
+    tuner = Tuner(cfg, SCHEDULE_MAPPING, batches=data, table_shapes=[(100, d) for d in dims],
+                  data_types=["float"] * 5, schedule_types=[[WarpPerSampleSchedule]] * 5)
+    mix = [c[0] for c in tuner.feat_sched_param_candidates]
+    emitted = {}
+    monkeypatch.setattr(Tuner, "emit_codes", lambda self, **kw: emitted.update(kw))
+    monkeypatch.setattr(Tuner, "_schedule_builds", lambda self, jobs, cfg: None)
+    ticks = [100.0, 300.0, 50.0, 70.0, 5000.0]      # kind (dim 16): 400, (dim 64): 120, (dim 32): 5000
+
+    def fake_ticks(lib, shapes, types, npzs, out, tb, xs, gpu_id=None):
+        os.makedirs(os.path.dirname(out), exist_ok=True)
+        with open(out, "w") as f:
+            f.write("".join(f"{t}\n" for t in ticks))
+    monkeypatch.setattr(tuner_mod, "measure_feature_ticks", fake_ticks)
+    tcfg = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=1, in_process=True)
+    # tile_bytes tiny enough that every feature gets one tile per bag-granule: equal tile counts
+    order = tuner.tile_time_order(mix, 4, 64, 16, tcfg)
+    assert emitted["timing"] is True and emitted["feat_schedules"] is mix
+    tiles = tiles_per_feature([d[0][1] for d in data], [d * 4 + 4 for d in dims], [d * 4 + 4 for d in dims],
+                              [s.TileGranularity(p) for s, p in mix], 64, grid_blocks=16)
+    per_kind = {16: (ticks[0] + ticks[1]) / (tiles[0] + tiles[1]), 64: (ticks[2] + ticks[3]) / (tiles[2] + tiles[3]),
+                32: ticks[4] / tiles[4]}
+    want = sorted(range(5), key=lambda f: (-per_kind[dims[f]], f))
+    assert order == want and order[0] == 4 and order.index(0) < order.index(1)
+    ticks[:] = [100.0, 100.0, 100.0, 100.0, 100.0]
+    tuner2 = Tuner(cfg, SCHEDULE_MAPPING, batches=data[:2] * 2 + data[:1], table_shapes=[(100, 16)] * 5,
+                   data_types=["float"] * 5, schedule_types=[[WarpPerSampleSchedule]] * 5)
+    assert tuner2.tile_time_order([c[0] for c in tuner2.feat_sched_param_candidates], 4, 64, 16, tcfg) is None
+
+
 def test_kernel_trace_parser_groups_calls_and_takes_medians(tmp_path):
     """rocprofv3 ``*_kernel_trace.csv``: a call is a FusedKnl dispatch plus the library's own
     kernels launched ahead of it; per batch the median over the passes after the warm-up pass."""
