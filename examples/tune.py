@@ -88,9 +88,10 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--walk_stage", choices=["auto", "on", "off"], default="auto",
                         help="after the global stage, try the winning mix with its features laid out in "
                              "the tile space by their time per tile, and with the last passes of the "
-                             "tile walk drawn from ticket counters, and keep what is faster on the "
-                             "samples; auto = for models of 256 features and more whose workgroups get fewer "
-                             "than eight tiles each")
+                             "tile walk (2, 8, all) drawn from ticket counters, and keep what is faster on the "
+                             "samples; auto = a drawn end for models whose workgroups get three tiles each "
+                             "or more, an order for models of 256 features and more whose workgroups "
+                             "get fewer than eight")
     parser.add_argument("--build_climb_trials", type=int, default=0,
                         help="global stage: that many single-feature variants of the winning mix are "
                              "built as production kernels and timed; the faster ones are adopted")
@@ -106,6 +107,9 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--incumbent", type=str,
                         help="schedule.json of an earlier tuning run of this model: one more contender of "
                              "the global stage (and the start of the build climb if it wins)")
+    parser.add_argument("--incumbent_only", action="store_true", default=False,
+                        help="global stage for the --incumbent mix alone (occupancy, traffic per tile, "
+                             "tile walk, outlier tiles): no tuning build, no other contender")
     parser.add_argument("--validate_clusters", action="store_true", default=False,
                         help="after tuning: build, for every cluster, the production kernel with and "
                              "without the cluster's fastest option and set the change beside the one "
@@ -210,17 +214,26 @@ def main():
     tune_config = create_tune_config(args)
 
     if args.compile_only:
-        if tune_config.interference == "model":
-            tuner.compile_tournament(tune_config)
-        else:
-            tuner.compile_local(tune_config)
-        # ... and the contenders of the global stage that are known without a measurement
-        tuner.compile_default_contenders(tune_config)
-        print(f"local-stage kernels built under {tuner.basic.codegen_dir}")
+        if not args.incumbent_only:
+            if tune_config.interference == "model":
+                tuner.compile_tournament(tune_config)
+            else:
+                tuner.compile_local(tune_config)
+            # ... and the contenders of the global stage that are known without a measurement
+            tuner.compile_default_contenders(tune_config)
+        tuner.compile_incumbent_contenders(tune_config)
+        print(f"kernels built under {tuner.basic.codegen_dir}")
         return
 
     if args.launch_only:
         occupancy, sched_params = tuner.solve_launch_only(tune_config)
+        print(occupancy, tuner.opt_tile_bytes, tuner.opt_xcd_segments)
+        return
+
+    if args.incumbent_only:
+        if not args.incumbent:
+            raise SystemExit("--incumbent_only needs --incumbent <schedule.json>")
+        occupancy, sched_params = tuner.solve_incumbent_only(tune_config)
         print(occupancy, tuner.opt_tile_bytes, tuner.opt_xcd_segments)
         return
 

@@ -40,6 +40,8 @@ def waves_per_simd(occupancy: int, block_threads: int) -> int:
 
 # XCDs (L2 slices) of an MI355X; workgroup i of a launch runs on XCD i % 8
 XCD_COUNT = 8
+# ``drawn_tail`` of a library all of whose tiles are drawn: more passes than any walk has
+DRAWN_ALL = 100000
 # per-bag traffic that does not depend on the bag length, besides the output slice: one offset
 BAG_FIXED_BYTES = 4
 INDEX_BYTES = 4
@@ -278,6 +280,7 @@ constexpr bool OUTLIERS = RFX_OUTLIERS;
 constexpr int MAX_LONG_DIM = {max_long_dim};
 // ... or, in their place in the workspace, the ticket counters of a drawn end of the tile walk
 #define RFX_DRAWN_TAIL {int(drawn_tail)}
+#define RFX_DRAWN_ALL {DRAWN_ALL}      // from this many passes on: every tile is drawn
 constexpr int DRAWN_TAIL = RFX_DRAWN_TAIL;
 static_assert(!(OUTLIERS && DRAWN_TAIL > 0), "one or the other");
 using OutlierSpace = {"rfx::TailTickets" if drawn_tail else f"rfx::OutlierSpace<MAX_LONG_DIM, {outlier_capacity(num_feats)}>"};
@@ -537,12 +540,26 @@ extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
   __syncthreads();
   if (threadIdx.x == 0) rfx::outliers_done(d_outliers);
 ''' if outliers else ''
+        drawn_begin = ''
         if drawn_tail:
+            # every tile drawn: a workgroup's first ticket does not wait for the binding
+            drawn_begin = '''
+  int first_ticket = 0;
+  if (DRAWN_TAIL >= RFX_DRAWN_ALL && threadIdx.x == 0)
+    first_ticket = rfx::draw_tail_ticket(d_outliers, xcd_segments > 0 && gridDim.x % XCDS == 0 ? blockIdx.x % XCDS : 0);
+'''
             loop_head = f'''  // The last DRAWN_TAIL passes of the walk are drawn: tickets of this workgroup's XCD (of the
-  // whole device for a flat walk) count on from static_last.
+  // whole device for a flat walk) count on from static_last.  A ticket is asked for one tile
+  // ahead, so that its round trip hides behind a tile's work -- except the first one after the
+  // dealt tiles, which a workgroup asks for only when those are done (asked for with its last
+  // dealt tile, a workgroup that is late would be bound to one more tile before it knows: a
+  // thousand features of five tiles per workgroup took 69.6 us that way, 68.6 us with the
+  // round trip in the open).  When every tile is drawn, the first ticket is asked for ahead
+  // of the binding.
   rfx::TailTickets *const d_tickets = d_outliers;
   __shared__ int s_ticket[2];
-  const int static_last = max(0, walk_last - DRAWN_TAIL * walk_step);
+  const int static_last = DRAWN_TAIL >= RFX_DRAWN_ALL ? 0 :
+      static_cast<int>(max(0ll, walk_last - static_cast<long long>(DRAWN_TAIL) * walk_step));
   int walk = walk_first, ticket_slot = 0, next_ticket = 0;
   bool drawing = false;
   for (;;) {{
@@ -553,15 +570,14 @@ extern "C" __global__ void __launch_bounds__(256) OutlierKnl(
         walk += walk_step;
       }} else {{
         drawing = true;
-        if (threadIdx.x == 0) s_ticket[0] = rfx::draw_tail_ticket(d_tickets, xcd);
+        if (threadIdx.x == 0)
+          s_ticket[0] = DRAWN_TAIL >= RFX_DRAWN_ALL ? first_ticket : rfx::draw_tail_ticket(d_tickets, xcd);
         continue;
       }}
     }} else {{
       __syncthreads();                         // the ticket is there, the previous tile is done
       at = static_last + s_ticket[ticket_slot];
       if (at >= walk_last) break;
-      // the next ticket: its value is needed only when this tile is done, so the round trip
-      // hides behind the tile
       if (threadIdx.x == 0) next_ticket = rfx::draw_tail_ticket(d_tickets, xcd);
       ticket_slot ^= 1;
     }}
@@ -628,7 +644,7 @@ extern "C" __global__ void {launch_bounds} FusedKnl(
     OutlierSpace *__restrict__ d_outliers, const int *__restrict__ d_lookup_counts) {{
 {bind_decl}
   __shared__ KnlTempStorage s;
-{stage_decl}{timing_init}
+{stage_decl}{timing_init}{drawn_begin}
   const rfx::IoView io{{d_io_ptrs, d_arg_buffers, d_arg_buffer_offsets, batch, d_lookup_counts, {"c_ext_feat" if tile_order is not None else "nullptr"}}};
 {bind_call}
 {timing_bound}

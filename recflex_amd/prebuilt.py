@@ -311,6 +311,14 @@ def _c3s_ordered() -> ModelSpec:
     return _ordered(spec, "c3s_ordered", 11, drawn_tail=2)
 
 
+def _drawn_all(spec: ModelSpec, name: str, **emit_kwargs) -> ModelSpec:
+    """The same model and schedules with every tile of the walk drawn from the ticket counters."""
+    from .code_emitter.codegen import DRAWN_ALL
+    kwargs = {k: v for k, v in spec.emit_kwargs.items() if k != "outliers"}
+    kwargs.update(drawn_tail=DRAWN_ALL, **emit_kwargs)
+    return spec._replace(workload=spec.workload._replace(name=name), emit_kwargs=kwargs)
+
+
 _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "c1": lambda: _default(make_workload("C1")),
     "c2": lambda: _default(make_workload("C2")),
@@ -345,6 +353,8 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "wide_ordered": lambda: _ordered(_wide(), "wide_ordered", 13, drawn_tail=1),
     "wider_ordered": lambda: _ordered(_wide(2500, "wider"), "wider_ordered", 14, drawn_tail=3),
     "onehots_ordered": lambda: _ordered(_onehots(), "onehots_ordered", 15, drawn_tail=8),
+    "c3s_drawn_all": lambda: _drawn_all(_c3s_outliers(), "c3s_drawn_all"),
+    "wide_drawn_all_flat": lambda: _drawn_all(_wide(), "wide_drawn_all_flat", xcd_aware=False),
     # fp16 and int8 tables with outlier tiles (integer-valued: sums exact)
     "c4s_outliers": lambda: _default(make_workload("C4", batch=128, num_features=48, max_rows=30_000)
                                      ._replace(name="c4s_outliers", table_values="integer"), outliers=True),

@@ -32,7 +32,7 @@ from typing import Dict, List, NamedTuple, Optional, Sequence, Tuple
 import numpy as np
 
 from recflex_amd.code_emitter import CodeEmitter, ScheduleBase, MetaData
-from recflex_amd.code_emitter.codegen import (BAG_FIXED_BYTES, DEFAULT_TILE_BYTES, INDEX_BYTES,
+from recflex_amd.code_emitter.codegen import (BAG_FIXED_BYTES, DEFAULT_TILE_BYTES, DRAWN_ALL, INDEX_BYTES,
                                                waves_per_simd)
 from recflex_amd.model_build import DEFAULT_XCD_SEGMENTS
 from recflex_amd.utils import compile_build, os_check
@@ -82,13 +82,20 @@ class TuneConfig(NamedTuple):
     outliers: Optional[bool] = None
     # undecided (None): kept only if the whole call is faster by this share on the samples
     outliers_min_gain: float = 0.02
-    # the order of the features in the kernel's tile space and a drawn end of the tile walk
-    # (Tuner.decide_walk): True / False, or None = tried for models of at least
+    # the tile walk (Tuner.decide_walk): a drawn end, and the order of the features in the
+    # kernel's tile space.  False: neither is tried; True: both; None: a drawn end on models
+    # whose workgroups get a few tiles each at least, an order on models of at least
     # ``walk_stage_min_feats`` features whose workgroups get fewer than
     # ``walk_stage_max_tiles`` tiles each on the samples (with more, the deal evens out by itself)
     walk_stage: Optional[bool] = None
     walk_stage_min_feats: int = 256
     walk_stage_max_tiles: float = 8.0
+    # passes drawn at the end of the walk that are tried (DRAWN_ALL: every tile), on models whose
+    # workgroups get at least ``walk_drawn_min_tiles`` tiles each on the samples
+    drawn_tail_candidates: Sequence[int] = (2, 8, DRAWN_ALL)
+    walk_drawn_min_tiles: float = 3.0
+    # segments per XCD a drawn winner is also timed with (those finer than its own)
+    walk_xcd_segments_candidates: Sequence[int] = (64, 128)
     walk_min_gain: float = 0.01
     # local-stage interference: "model" = every candidate of every feature is compiled into one
     # kernel of the whole model and timed while all other features run beside it;
@@ -154,6 +161,8 @@ class TuneConfig(NamedTuple):
     # as ``solve`` writes it), timed as one more contender at every occupancy: a model that is
     # tuned again starts from what it has
     incumbent: Optional[str] = None
+    # the incumbent is the only contender of the global stage (Tuner.solve_incumbent_only)
+    only_incumbent: bool = False
 
 
 def padded_sched_num(orig_num: int, max_concurrent_blocks: int) -> int:
@@ -172,6 +181,7 @@ def pick_launch_option(launch_opts: List[Tuple[int, int]], times: List[float],
     limit = times[best] * (1.0 + tolerance)
     near = [k for k, (_, xs) in enumerate(launch_opts) if xs > 0 and times[k] <= limit]
     return min(near, key=lambda k: (launch_opts[k][1], times[k]))
+
 
 
 def release_device_memory() -> None:
@@ -1006,6 +1016,16 @@ class Tuner:
                                        grid_blocks=tune_config.sm_count * occupancy)
         return tiles
 
+    def _build_walk_timing(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
+                           tile_bytes: int, xcd_segments: int, tune_config: TuneConfig) -> str:
+        """Emit and build the mix with tick counters per feature; returns its directory."""
+        output_dir = f"{self.basic.codegen_dir}/walk_timing/o{occupancy}"
+        self.emit_codes(output_dir=output_dir, feat_schedules=sched_params, occupancy=occupancy,
+                        inline=tune_config.inline, timing=True, debug=tune_config.debug,
+                        tile_bytes=tile_bytes, xcd_segments=max(xcd_segments, 0))
+        self._schedule_builds([(output_dir, f"{output_dir}/build")], tune_config)
+        return output_dir
+
     def tile_time_order(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
                         tile_bytes: int, xcd_segments: int, tune_config: TuneConfig
                         ) -> Optional[List[int]]:
@@ -1014,11 +1034,7 @@ class Tuner:
         feature's ticks are divided by the tiles the binding gives it.  (The tournament's tile
         times do not serve: its kernel holds every candidate, and an order by its figures was no
         better than the model's own.)  None if nothing can be told apart."""
-        output_dir = f"{self.basic.codegen_dir}/walk_timing/o{occupancy}"
-        self.emit_codes(output_dir=output_dir, feat_schedules=sched_params, occupancy=occupancy,
-                        inline=tune_config.inline, timing=True, debug=tune_config.debug,
-                        tile_bytes=tile_bytes, xcd_segments=max(xcd_segments, 0))
-        self._schedule_builds([(output_dir, f"{output_dir}/build")], tune_config)
+        output_dir = self._build_walk_timing(sched_params, occupancy, tile_bytes, xcd_segments, tune_config)
         result = f"{output_dir}/feature_ticks.txt"
         if os.path.exists(result):
             os.remove(result)
@@ -1050,31 +1066,17 @@ class Tuner:
             return None
         return sorted(range(self.num_feats), key=lambda f: (-per_tile[f], f))
 
-    def decide_walk(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
-                    measured_times: Dict[int, Dict[int, List[float]]], tile_bytes: int,
-                    xcd_segments: int, outliers: bool, tune_config: TuneConfig
-                    ) -> Tuple[Optional[List[int]], int]:
-        """(tile_order, drawn_tail) for ``optimal/``, by measurement.  With the features sorted
-        by their time per tile, the strided deal hands every workgroup one tile of each kind,
-        and a drawn end then has cheap tiles to fill it with: worth 5 and 9 % on a model of a
-        thousand small features whose workgroups get five tiles each, nothing on one of a
-        hundred features and ten tiles per workgroup.  The mix is built as it is, ordered, and
-        ordered with the last two passes drawn, all three are timed on the samples like
-        contenders of the global stage, and a variant is kept if it gains
-        ``TuneConfig.walk_min_gain``."""
-        want = tune_config.walk_stage
-        if want is None and self.num_feats >= tune_config.walk_stage_min_feats:
-            batches = getattr(self, "batches", None) or [[]]
-            per_workgroup = (self.sample_tiles(sched_params, occupancy, tile_bytes, tune_config).sum()
-                             / max(1, len(batches[0])) / (tune_config.sm_count * occupancy))
-            want = per_workgroup < tune_config.walk_stage_max_tiles
-        order = (self.tile_time_order(sched_params, occupancy, tile_bytes, xcd_segments, tune_config)
-                 if want else None)
-        if order is None:
-            return None, 0
-        variants = {"as_is": (None, 0), "ordered": (order, 0)}
-        if not outliers:
-            variants["ordered_drawn"] = (order, 2)
+    @staticmethod
+    def _drawn_variants(tune_config: TuneConfig) -> Dict[str, Tuple[None, int]]:
+        return {"drawn_all" if n >= DRAWN_ALL else f"drawn_{n}": (None, int(n))
+                for n in tune_config.drawn_tail_candidates}
+
+    def _build_walk_variants(self, variants: Dict[str, Tuple[Optional[List[int]], int]],
+                             sched_params: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
+                             tile_bytes: int, xcd_segments: int, outliers: bool,
+                             tune_config: TuneConfig) -> Dict[str, str]:
+        """Emit and build ``walk_{name}/o{occ}`` for every variant (tile_order, drawn_tail);
+        returns their directories."""
         dirs = {name: f"{self.basic.codegen_dir}/walk_{name}/o{occupancy}" for name in variants}
         jobs = []
         for name, (tile_order, drawn_tail) in variants.items():
@@ -1084,24 +1086,88 @@ class Tuner:
                             tile_order=tile_order, drawn_tail=drawn_tail)
             jobs.append((dirs[name], f"{dirs[name]}/build"))
         self._schedule_builds(jobs, tune_config)
-        manager = self._measure_manager(tune_config)
-        if tune_config.profiler == "rocprofv3" or manager:
-            release_device_memory()
+        return dirs
+
+    def decide_walk(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
+                    measured_times: Dict[int, Dict[int, List[float]]], tile_bytes: int,
+                    xcd_segments: int, outliers: bool, tune_config: TuneConfig
+                    ) -> Tuple[Optional[List[int]], int, int]:
+        """(tile_order, drawn_tail, xcd_segments) for ``optimal/``, by measurement.
+
+        A drawn end: the last passes of the tile walk -- or all of them -- are drawn from ticket
+        counters instead of dealt out.  Workgroups whose tiles were cheap then take more of them,
+        and the workgroups of an XCD stay together on neighbouring tiles, i.e. on the hot rows
+        of one or two features at a time: 8-11 % on a model of 400 features and 80 tiles per
+        workgroup, 3.5 % on one of 200 features with eight passes drawn (all of them: 2 %), a
+        loss of 1-3 % on one of 100 features and 14 short tiles per workgroup.  Tried with
+        ``TuneConfig.drawn_tail_candidates`` when the workgroups get at least
+        ``walk_drawn_min_tiles`` tiles each and the library has no outlier tiles (which are
+        drawn already).
+
+        An order: with the features sorted by their time per tile, the strided deal hands every
+        workgroup one tile of each kind, and a drawn end has cheap tiles to fill it with: 3 and
+        7 % on a model of a thousand small features whose workgroups get five tiles each,
+        nothing at ten tiles per workgroup.  Tried on wide models of few tiles per workgroup.
+
+        All variants are built, timed on the samples like contenders of the global stage, and
+        the fastest is kept if it gains ``TuneConfig.walk_min_gain``.  A drawn winner is then
+        timed with finer segments per XCD (``walk_xcd_segments_candidates``): drawing takes care
+        of the balance inside an XCD, finer segments of the balance between them."""
+        keep_as_is = (None, 0, xcd_segments)
+        if tune_config.walk_stage is False:
+            return keep_as_is
+        batches = getattr(self, "batches", None) or [[]]
+        per_workgroup = (self.sample_tiles(sched_params, occupancy, tile_bytes, tune_config).sum()
+                         / max(1, len(batches[0])) / (tune_config.sm_count * occupancy))
+        forced = tune_config.walk_stage is True
+        variants = {"as_is": (None, 0)}
+        if not outliers and (forced or per_workgroup >= tune_config.walk_drawn_min_tiles):
+            variants.update(self._drawn_variants(tune_config))
+        order = None
+        if forced or (self.num_feats >= tune_config.walk_stage_min_feats
+                      and per_workgroup < tune_config.walk_stage_max_tiles):
+            order = self.tile_time_order(sched_params, occupancy, tile_bytes, xcd_segments, tune_config)
+        if order is not None:
+            variants["ordered"] = (order, 0)
+            if not outliers:
+                variants["ordered_drawn_2"] = (order, 2)
+        if len(variants) == 1:
+            return keep_as_is
+        dirs = self._build_walk_variants(variants, sched_params, occupancy, tile_bytes, xcd_segments,
+                                         outliers, tune_config)
         cfg = tune_config._replace(remeasure=True)
-        for output_dir in dirs.values():
-            self._kernel_time(output_dir, cfg, manager)
-        if manager:
-            manager.join()
-        times = {name: self._read_kernel_time(dirs[name], tune_config) for name in variants}
+
+        def timed(runs: List[Tuple[str, int]]) -> List[float]:
+            manager = self._measure_manager(tune_config)
+            if tune_config.profiler == "rocprofv3" or manager:
+                release_device_memory()
+            for output_dir, xs in runs:
+                self._kernel_time(output_dir, cfg, manager, 0, xs)
+            if manager:
+                manager.join()
+            return [self._read_kernel_time(output_dir, tune_config, 0, xs) for output_dir, xs in runs]
+
+        times = dict(zip(variants, timed([(dirs[name], 0) for name in variants])))
         best = min(times, key=times.get)
         keep = best if times[best] < times["as_is"] * (1.0 - tune_config.walk_min_gain) else "as_is"
         print("tile walk: " + ", ".join(f"{name} {t:.0f} ns" for name, t in times.items())
               + f": {keep.replace('_', ' ')}", flush=True)
-        return variants[keep]
+        tile_order, drawn_tail = variants[keep]
+        if drawn_tail and xcd_segments > 0:
+            finer = [xs for xs in tune_config.walk_xcd_segments_candidates if xs > xcd_segments]
+            if finer:
+                finer_times = timed([(dirs[keep], xs) for xs in finer])
+                k = int(np.argmin(finer_times))
+                print(f"tile walk, segments per XCD: {xcd_segments}: {times[keep]:.0f} ns, "
+                      + ", ".join(f"{xs}: {t:.0f} ns" for xs, t in zip(finer, finer_times)), flush=True)
+                if finer_times[k] < times[keep] * (1.0 - tune_config.walk_min_gain):
+                    xcd_segments = finer[k]
+        return tile_order, drawn_tail, xcd_segments
 
     def solve(self, measured_times: Dict[int, Dict[int, List[float]]],
               tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
-        occu_opt_sched_params = self.select_per_occupancy(measured_times, tune_config.occupancies)
+        occu_opt_sched_params = ([] if tune_config.only_incumbent else
+                                 self.select_per_occupancy(measured_times, tune_config.occupancies))
         opt_occupancy, opt_sched_params = self.tune_occupancy(occu_opt_sched_params, tune_config)
         output_dir = self.opt_output_dir
         optimal = f"{self.basic.codegen_dir}/optimal"
@@ -1121,8 +1187,9 @@ class Tuner:
         if outliers is None:
             outliers = self.decide_outliers(opt_sched_params, opt_occupancy, tile_bytes, xcd_segments,
                                             tune_config)
-        tile_order, drawn_tail = self.decide_walk(opt_sched_params, opt_occupancy, measured_times,
-                                                  tile_bytes, xcd_segments, bool(outliers), tune_config)
+        tile_order, drawn_tail, xcd_segments = self.decide_walk(
+            opt_sched_params, opt_occupancy, measured_times, tile_bytes, xcd_segments, bool(outliers),
+            tune_config)
         # a contender whose library came out of the compile cache (the same source had been built
         # in another directory) has no host module of its own: optimal/ is then built in place
         import glob
@@ -1153,6 +1220,15 @@ class Tuner:
                              for c in self.feat_sched_param_candidates[f]]
                        for occ in cfg.occupancies} for f in range(self.num_feats)}
         return self.solve(results, cfg)
+
+    def solve_incumbent_only(self, tune_config: TuneConfig) -> Tuple[int, List[Tuple[ScheduleBase, NamedTuple]]]:
+        """Global stage for the mix of ``TuneConfig.incumbent`` alone: swept over occupancy,
+        traffic per tile and tile walk, then the decisions on outlier tiles and on the walk.
+        Needs no tuning build; ends like ``solve`` with ``optimal/``."""
+        if not tune_config.incumbent:
+            raise ValueError("no incumbent given")
+        return self.solve({}, tune_config._replace(include_default=False, only_incumbent=True,
+                                                   build_climb_trials=0))
 
     def _build_full(self, output_dir: str, sched_params, occupancy: Optional[int],
                     tune_config: TuneConfig, fixed_task_block_nums: List[int] = None,
@@ -1234,6 +1310,42 @@ class Tuner:
         return [(f"{self.basic.codegen_dir}/default/o{occupancy}", occupancy, default_mix)
                 for occupancy in tune_config.occupancies]
 
+    def incumbent_contenders(self, tune_config: TuneConfig) -> list:
+        """(directory, occupancy, schedules) of the mix in ``TuneConfig.incumbent`` at every
+        occupancy."""
+        if not tune_config.incumbent:
+            return []
+        from recflex_amd.schedules import schedule_from_config
+        with open(tune_config.incumbent) as f:
+            doc = json.load(f)
+        entries = doc["schedules"] if isinstance(doc, dict) else doc
+        if len(entries) != self.num_feats:
+            raise ValueError(f"{tune_config.incumbent} describes {len(entries)} features, the model has {self.num_feats}")
+        mix = [schedule_from_config(e, meta, self.basic.block_threads) for e, meta in zip(entries, self.metas)]
+        return [(f"{self.basic.codegen_dir}/incumbent/o{occupancy}", occupancy, mix)
+                for occupancy in tune_config.occupancies]
+
+    def compile_incumbent_contenders(self, tune_config: TuneConfig) -> None:
+        """Emit and build ``incumbent/o{occ}`` (no GPU needed) and, where the launch options are
+        given rather than swept (one candidate each), the drawn-end variants of the walk stage
+        and its timing build, so that a run with ``only_incumbent`` finds them built."""
+        contenders = self.incumbent_contenders(tune_config)
+        jobs = []
+        for output_dir, occupancy, sched_params in contenders:
+            if self._build_full(output_dir, sched_params, occupancy, tune_config):
+                jobs.append((output_dir, f"{output_dir}/build"))
+        self._schedule_builds(jobs, tune_config)
+        tile_opts = list(tune_config.tile_bytes_candidates) or [0]
+        walk_opts = list(tune_config.xcd_segments_candidates) or [0]
+        if tune_config.walk_stage is False or len(tile_opts) != 1 or len(walk_opts) != 1:
+            return
+        tile_bytes, xcd_segments = tile_opts[0] or tune_config.tile_bytes, walk_opts[0]
+        for _, occupancy, sched_params in contenders:
+            variants = dict({"as_is": (None, 0)}, **self._drawn_variants(tune_config))
+            self._build_walk_variants(variants, sched_params, occupancy, tile_bytes, xcd_segments, False,
+                                      tune_config)
+            self._build_walk_timing(sched_params, occupancy, tile_bytes, xcd_segments, tune_config)
+
     def compile_default_contenders(self, tune_config: TuneConfig) -> None:
         """Emit and build ``default/o{occ}`` (no GPU needed)."""
         jobs = []
@@ -1249,16 +1361,7 @@ class Tuner:
         for occupancy, sched_params in zip(tune_config.occupancies, occu_opt_sched_params):
             contenders.append((self.get_output_build_dir(-1, occupancy)[0], occupancy, sched_params))
         contenders += self.default_contenders(tune_config)
-        if tune_config.incumbent:
-            from recflex_amd.schedules import schedule_from_config
-            with open(tune_config.incumbent) as f:
-                doc = json.load(f)
-            entries = doc["schedules"] if isinstance(doc, dict) else doc
-            if len(entries) != self.num_feats:
-                raise ValueError(f"{tune_config.incumbent} describes {len(entries)} features, the model has {self.num_feats}")
-            mix = [schedule_from_config(e, meta, self.basic.block_threads) for e, meta in zip(entries, self.metas)]
-            for occupancy in tune_config.occupancies:
-                contenders.append((f"{self.basic.codegen_dir}/incumbent/o{occupancy}", occupancy, mix))
+        contenders += self.incumbent_contenders(tune_config)
 
         jobs = []
         for output_dir, occupancy, sched_params in contenders:
