@@ -69,7 +69,9 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--occupancies", type=str, help="comma-separated workgroups per CU to try")
     parser.add_argument("--sample_batch_nums", type=int, default=128)
     parser.add_argument("--profiler", type=str, default="rocprofv3", choices=["rocprofv3", "events"])
-    parser.add_argument("--tile_bytes", type=int, default=0)
+    parser.add_argument("--tile_bytes", type=str, default="",
+                        help="traffic per tile of the tuning builds and contenders (bytes; default 65536); "
+                             "auto = sized by the device from every batch, as untuned builds do")
     parser.add_argument("--tile_bytes_candidates", type=str,
                         help="comma-separated traffic-per-tile values swept in the global stage")
     parser.add_argument("--xcd_segments_candidates", type=str,
@@ -195,7 +197,7 @@ def create_tune_config(args: argparse.Namespace) -> TuneConfig:
               "climb_passes": args.climb_passes, "outliers": {"auto": None, "on": True, "off": False}[args.outliers],
               "walk_stage": {"auto": None, "on": True, "off": False}[args.walk_stage]}
     if args.tile_bytes:
-        kwargs["tile_bytes"] = args.tile_bytes
+        kwargs["tile_bytes"] = 0 if args.tile_bytes == "auto" else int(args.tile_bytes)
     if args.xcd_segments_candidates:
         kwargs["xcd_segments_candidates"] = [int(v) for v in args.xcd_segments_candidates.split(",")]
     if args.launch_time_tolerance:

@@ -44,7 +44,8 @@ its library is missing.  Names:
                    more than the static array of ``recom_process_static_workspace`` may hold
 ``refa``, ``reff4`` models shaped like the reference's example models A and a quarter of F (1 000 and
                    2 500 small features, batch 256; ``workloads.REF_SHAPED``), default schedules;
-                   ``refa_tuned``: with ``tuned/refa_schedule.json`` if that file exists
+                   ``refa_tuned`` / ``reff4_tuned``: with ``tuned/refa_schedule.json`` /
+                   ``tuned/reff4_schedule.json`` if that file exists
 ``wide``           1 500 small features (several binding rounds per thread)
 ``wider``          2 500 small features (bound once per launch by the binding kernel)
 """
@@ -378,6 +379,7 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "refa": lambda: _default(make_workload("REFA")),
     "reff4": lambda: _default(make_workload("REFF4")),
     "refa_tuned": lambda: _tuned(make_workload("REFA"), "refa_schedule.json"),
+    "reff4_tuned": lambda: _tuned(make_workload("REFF4"), "reff4_schedule.json"),
     "b128": lambda: _other_block_size(128),
     "b512": lambda: _other_block_size(512),
 }

@@ -557,9 +557,11 @@ def tiles_per_feature(offsets: Sequence[np.ndarray], lookup_bytes: Sequence[int]
     for this batch on a grid of ``grid_blocks`` workgroups (0: unknown, taken as too large for
     the whole-pass rule of plentiful tiles to apply).  A schedule that can split bags over
     workgroups (granularity -1) counts as one bag per workgroup pass: a binding frozen at emit
-    time never splits."""
+    time never splits.  ``tile_bytes`` <= 0: the size the device picks for this batch."""
     out = []
     num_feats = len(offsets)
+    if tile_bytes <= 0:
+        tile_bytes = auto_tile_bytes(offsets, lookup_bytes, bag_bytes, grid_blocks)
     for off, lb, bb, g in zip(offsets, lookup_bytes, bag_bytes, gran):
         g = 1 if g < 0 else g
         batch = len(off) - 1

@@ -74,6 +74,8 @@ class TuneConfig(NamedTuple):
     profiler: str = "rocprofv3"
     # run measurement workers in this process instead of one spawned process per measurement
     in_process: bool = True
+    # traffic a tile carries in the tuning builds and contenders; 0 = sized by the device from
+    # every batch (rfx::auto_tile_size), as untuned builds do
     tile_bytes: int = DEFAULT_TILE_BYTES
     # emit optimal/ with outlier tiles: bags far beyond their schedule's reach are found by a pass
     # over the offsets ahead of the fused kernel and summed by several workgroups (skewed data).
@@ -92,7 +94,7 @@ class TuneConfig(NamedTuple):
     walk_stage_max_tiles: float = 8.0
     # passes drawn at the end of the walk that are tried (DRAWN_ALL: every tile), on models whose
     # workgroups get at least ``walk_drawn_min_tiles`` tiles each on the samples
-    drawn_tail_candidates: Sequence[int] = (2, 8, DRAWN_ALL)
+    drawn_tail_candidates: Sequence[int] = (2, 4, 8, DRAWN_ALL)
     walk_drawn_min_tiles: float = 3.0
     # segments per XCD a drawn winner is also timed with (those finer than its own)
     walk_xcd_segments_candidates: Sequence[int] = (64, 128)

@@ -155,6 +155,11 @@ def test_host_binding_restatement():
     assert tiles_per_feature([off], [132], [132], [1024], 65536) == [46]   # ceil(2048/45)
     # a pass of 256 bags = 372 KB <= 8 x 64 KiB: whole passes
     assert tiles_per_feature([off], [132], [132], [256], 65536) == [8]
+    # no tile size given: the one the device would pick for this batch and grid
+    from recflex_amd.tuning.measure import auto_tile_bytes
+    auto = auto_tile_bytes([off], [132], [132], 16)
+    assert tiles_per_feature([off], [132], [132], [16], 0, grid_blocks=16) == \
+        tiles_per_feature([off], [132], [132], [16], auto, grid_blocks=16)
     assert tiles_per_feature([off], [132], [132], [1024], 1024) == [2048]  # never more than bags
     assert tiles_per_feature([off], [132], [132], [16], 1 << 30) == [1]
     empty = np.zeros(1, dtype=np.int32)
@@ -410,7 +415,7 @@ def test_tile_walk_is_decided_by_measurement(tmp_path, monkeypatch):
     assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, cfg._replace(walk_stage=False)) == (None, 0, 16)
     assert not built
     on = cfg._replace(walk_stage=True)
-    names = ["as_is", "drawn_2", "drawn_8", "drawn_all", "ordered", "ordered_drawn_2"]
+    names = ["as_is", "drawn_2", "drawn_4", "drawn_8", "drawn_all", "ordered", "ordered_drawn_2"]
     times.update(dict.fromkeys(names, 1000.0))
     times.update(ordered=940.0, ordered_drawn_2=900.0)
     times.update({("ordered_drawn_2", 64): 905.0, ("ordered_drawn_2", 128): 895.0})   # within the margin
@@ -443,7 +448,7 @@ def test_tile_walk_is_decided_by_measurement(tmp_path, monkeypatch):
     times.update(drawn_8=900.0)
     times.update({("drawn_8", 64): 950.0, ("drawn_8", 128): 960.0})
     assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, few) == (None, 8, 16)
-    assert [d.split("/walk_")[1].split("/")[0] for d in built] == ["as_is", "drawn_2", "drawn_8", "drawn_all"]
+    assert [d.split("/walk_")[1].split("/")[0] for d in built] == ["as_is", "drawn_2", "drawn_4", "drawn_8", "drawn_all"]
     del built[:]
     assert tuner.decide_walk(mix, 4, measured, 65536, 16, True, few) == (None, 0, 16) and not built
     wide = cfg._replace(walk_stage_min_feats=2, walk_stage_max_tiles=1e9)
