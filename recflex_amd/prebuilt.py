@@ -48,6 +48,8 @@ its library is missing.  Names:
                    ``tuned/reff4_schedule.json`` if that file exists
 ``wide``           1 500 small features (several binding rounds per thread)
 ``wider``          2 500 small features (bound once per launch by the binding kernel)
+``widest``         4 500 small features (more than 64 chunks of 64 features: the prefix sum's second
+                   level and the feature search walk their first level in two rounds)
 """
 
 import json
@@ -375,6 +377,7 @@ _SPECS: Dict[str, Callable[[], ModelSpec]] = {
     "manysplit": _many_split,
     "wide": _wide,
     "wider": lambda: _wide(2500, "wider"),
+    "widest": lambda: _wide(4500, "widest"),
     # models shaped like the reference's own examples (workloads.REF_SHAPED), default schedules
     "refa": lambda: _default(make_workload("REFA")),
     "reff4": lambda: _default(make_workload("REFF4")),

@@ -68,7 +68,7 @@ def test_binding_is_result_invariant(tile_bytes, grid, xcd):
     _assert_parity(*_run_model("c3s", tile_bytes=tile_bytes, grid_blocks=grid, xcd_segments=xcd))
 
 
-@pytest.mark.parametrize("name", ["variants", "edge", "onehots", "wide", "wider", "longbags"])
+@pytest.mark.parametrize("name", ["variants", "edge", "onehots", "wide", "wider", "widest", "longbags"])
 def test_integer_tables_are_bit_exact(name):
     """Integer-valued tables make every fp32 sum exact, so each schedule variant (any lane
     split, any reduction tree) must reproduce the oracle's bits."""
