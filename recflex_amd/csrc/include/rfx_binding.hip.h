@@ -212,15 +212,26 @@ __device__ __forceinline__ float wave_sum(float v) {
 // candidate f and the candidate tables are not read to find that out.
 // Returns the total number of tiles.  Ends with a barrier.
 //
-// Tile counts come from quotients of traffic figures; those are taken in single precision (a
+// A feature's traffic and the tile counts that follow from it are single-precision figures (a
 // 64-bit integer division costs some hundred instructions, and every workgroup of every launch
-// pays for the binding before its first load).  Being off by one tile near a boundary changes
-// nothing but the balance, and every workgroup computes the same figures.  The divisions that
-// decide which bags a tile holds stay exact.
-__device__ __forceinline__ long long approx_ceil_div(const long long a, const long long b) {
-  const float q = static_cast<float>(a) / static_cast<float>(b);
-  return static_cast<long long>(ceilf(q));
+// pays for the binding before its first load: at four features per thread and four workgroups
+// per CU the binding's 740 vector instructions kept every SIMD busy for 5 us).  Being off by
+// one tile near a boundary changes nothing but the balance, and every workgroup computes the
+// same figures.  The divisions that decide which bags a tile holds stay exact.
+//
+// a / b, exact, for 0 <= a < 2^22 and b >= 1: a single-precision quotient and one step of
+// correction either way, a third of the instructions of the 32-bit integer division.  The
+// binding takes four quotients per feature that decide which bags a tile holds and must be
+// exact; every workgroup of every launch computes them for all features before its first load.
+__device__ __forceinline__ int div_small(const int a, const int b) {
+  int q = static_cast<int>(static_cast<float>(a) * __builtin_amdgcn_rcpf(static_cast<float>(b)));
+  const int r = a - q * b;
+  q += r >= b ? 1 : 0;
+  q -= r < 0 ? 1 : 0;
+  return q;
 }
+// batches up to which div_small serves (its dividends stay below twice the batch)
+constexpr int kSmallDivBatch = 1 << 21;
 
 template <int F, int BT, bool SPLIT = false, bool ONE_CAND = false>
 __device__ __forceinline__ int
@@ -237,7 +248,7 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
   // up to 64 features: all of them sit in the first wavefront, which then needs no LDS and no
   // barrier to add up the traffic and to scan the tile counts
   constexpr bool ONE_WAVE = F <= 64;
-  long long cost[K];        // traffic of the feature in this batch
+  float cost[K];            // traffic of the feature in this batch (sizes tiles: 24 bits serve)
   int gran[K];              // bags per workgroup pass of the feature's schedule (kSplitGran: splits)
 
   // Step 1, the only one that reads memory, in two rounds of loads: the addresses, the schedule
@@ -249,7 +260,9 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     // surplus threads repeat the last feature, stores included: no branch stands between the
     // loads of this step
     const int f = min(tid + k * BT, F - 1);
-    io.addrs(f, idx_at[k], offs_at[k]);
+    idx_at[k] = offs_at[k] = 0;
+    // (a model that finds its addresses per tile and gets the lookup counts needs none here)
+    if (BindingStorage<F>::kKeepAddrs || !io.counts) io.addrs(f, idx_at[k], offs_at[k]);
     table_at[k] = 0;
     // (the once-per-launch binding kernel has no use for the tables' addresses and passes none)
     if constexpr (BindingStorage<F>::kKeepAddrs) table_at[k] = table_ptrs ? table_ptrs[io.ext_of(f)] : 0;
@@ -270,20 +283,21 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
   for (int k = 0; k < K; ++k) {
     const bool real = tid + k * BT < F;
     const int f = min(tid + k * BT, F - 1);
-    cost[k] = 0;
+    cost[k] = 0.f;
     bool one_per_bag = false;
     if (!fixed_tiles) {
       int first_lookup = 0;
-      int64_t lookups;
+      int lookups;
       if (io.counts) {                        // one array for all features instead of a line each
         lookups = io.count(f);
       } else {
         const int *offs = global_ptr<int>(offs_at[k]);
         first_lookup = offs[0];
-        lookups = static_cast<int64_t>(offs[B]) - first_lookup;
+        lookups = offs[B] - first_lookup;
       }
-      cost[k] = lookups * lookup_b[k] + static_cast<int64_t>(B) * bag_b[k];
-      traffic += real ? static_cast<float>(cost[k]) : 0.f;
+      cost[k] = static_cast<float>(lookups) * static_cast<float>(lookup_b[k]) +
+                static_cast<float>(B) * static_cast<float>(bag_b[k]);
+      traffic += real ? cost[k] : 0.f;
       one_per_bag = lookups == B && first_lookup == 0;
     }
     s.cand[f] = cand[k];
@@ -310,6 +324,8 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
       total = 0.f;
       for (int w = 0; w < BT / 64; ++w) total += partial[w];
     }
+    // the same in every lane: what follows from it is scalar arithmetic
+    total = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(total)));
     const long long total_bytes = static_cast<long long>(total);
     if (automatic) tile_size = auto_tile_size(total_bytes, grid_blocks);
     if (SPLIT) {
@@ -329,7 +345,16 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     }
   }
 
-  // Step 3: tiles of every feature, from registers.
+  // Step 3: tiles of every feature, from registers.  Traffic figures in single precision;
+  // the quotients that decide which bags a tile holds exact.
+  const float tile_f = static_cast<float>(tile_size);
+  const float inv_tile = __builtin_amdgcn_rcpf(tile_f);
+  const float inv_batch = B > 0 ? __builtin_amdgcn_rcpf(static_cast<float>(B)) : 0.f;
+  const float split_unit_f = static_cast<float>(split_unit);
+  const bool small = B < kSmallDivBatch;
+  // "tiles in plenty" below: (B / g) * F >= kPlentyTilesPerWorkgroup * grid  <=>  B >= g * need
+  const int plenty_need = grid_blocks > 0
+      ? static_cast<int>((static_cast<long long>(kPlentyTilesPerWorkgroup) * grid_blocks + F - 1) / F) : 0;
   int tiles_of[K];
 #pragma unroll
   for (int k = 0; k < K; ++k) {
@@ -338,25 +363,29 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     int g = gran[k];
     const bool may_split = g == kSplitGran && !fixed_tiles;
     if (g == kSplitGran) g = 1;
-    const int64_t want = fixed_tiles ? fixed_tiles[f] : approx_ceil_div(cost[k], tile_size);
     // mean traffic of one bag of this feature
-    const int64_t bag_cost = B > 0 ? static_cast<int64_t>(static_cast<float>(cost[k]) /
-                                                          static_cast<float>(B)) : 0;
-    int tiles = want < 1 ? 1 : (want > B ? B : static_cast<int>(want));
+    const float bag_cost = cost[k] * inv_batch;
+    int tiles;
+    if (fixed_tiles) {
+      const int want = fixed_tiles[f];
+      tiles = want < 1 ? 1 : (want > B ? B : want);
+    } else {
+      const float want = ceilf(cost[k] * inv_tile);
+      tiles = static_cast<int>(fminf(fmaxf(want, 1.f), static_cast<float>(B)));
+    }
     int bpt = 0;
-    int64_t parts = 1;
+    int parts = 1;
     // a bag is split from 1.25 units on (128 x 2 500 lookups: 102.8 us with bags of 1.7 units left
     // whole beside split ones, 89.3 us with those in two parts)
-    if (SPLIT && may_split && B > 0 && split_unit > 0 && 4 * bag_cost > 5 * split_unit) {
-      parts = approx_ceil_div(bag_cost, split_unit);
-      if (parts > kBindMaxParts) parts = kBindMaxParts;
-      if (parts * B > kBindMaxSplitTiles) parts = kBindMaxSplitTiles / B;
+    if (SPLIT && may_split && B > 0 && split_unit > 0 && 4.f * bag_cost > 5.f * split_unit_f) {
+      parts = static_cast<int>(fminf(ceilf(bag_cost / split_unit_f), static_cast<float>(kBindMaxParts)));
+      if (static_cast<long long>(parts) * B > kBindMaxSplitTiles) parts = kBindMaxSplitTiles / B;
     }
     if (parts > 1) {
-      tiles = B * static_cast<int>(parts);
-      bpt = -static_cast<int>(parts);
+      tiles = B * parts;
+      bpt = -parts;
     } else if (B > 0) {
-      bpt = (B + tiles - 1) / tiles;
+      bpt = small ? div_small(B + tiles - 1, tiles) : (B + tiles - 1) / tiles;
       // Tiles are whole workgroup passes (g bags) -- unless one pass of this schedule is more
       // than kMaxTileFactor times the traffic a tile should carry AND whole passes would leave
       // the grid short of tiles: then the tile keeps its share of the traffic and some of the
@@ -365,14 +394,14 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
       // least kPlentyTilesPerWorkgroup tiles per workgroup of the grid -- idle teams are a pure
       // loss: a batch whose bags are twice as long as the tile size was chosen for ran 262 us
       // with a quarter of the wavefronts busy in the long-bag features, 197 us with whole passes.
-      const int whole = (bpt + g - 1) / g * g;
+      const int passes = small ? div_small(bpt + g - 1, g) : (bpt + g - 1) / g;
+      const int whole = passes * g;
       const bool plenty = grid_blocks > 0 &&
-                          static_cast<int64_t>(B / g) * F >=
-                              static_cast<int64_t>(kPlentyTilesPerWorkgroup) * grid_blocks;
+                          static_cast<long long>(B) >= static_cast<long long>(g) * plenty_need;
       if (fixed_tiles || bpt >= g || plenty ||
-          static_cast<int64_t>(whole) * bag_cost <= static_cast<int64_t>(kMaxTileFactor) * tile_size)
+          static_cast<float>(whole) * bag_cost <= static_cast<float>(kMaxTileFactor) * tile_f)
         bpt = whole;
-      tiles = (B + bpt - 1) / bpt;
+      tiles = small ? div_small(B + bpt - 1, bpt) : (B + bpt - 1) / bpt;
     } else {
       tiles = 0;
     }
