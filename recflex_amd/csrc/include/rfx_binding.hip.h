@@ -63,8 +63,11 @@ struct IoView {
   // Both addresses of feature f from two independent loads of one cache line, whichever form the
   // inputs have (no branch: the binding issues these loads for all features at once).
   __device__ __forceinline__ void addrs(int f, int64_t &indices_at, int64_t &offsets_at) const {
+    addrs_at(ext_of(f), indices_at, offsets_at);
+  }
+  // ... of the feature the caller numbers f
+  __device__ __forceinline__ void addrs_at(const int f, int64_t &indices_at, int64_t &offsets_at) const {
     typedef long long pair_t __attribute__((ext_vector_type(2), aligned(8)));
-    f = ext_of(f);
     const bool ptrs = io_ptrs != nullptr;
     // pointer table: {indices, offsets} of f; packed form: {byte offset of f, of f + 1}
     const int64_t *src = ptrs ? io_ptrs + 2 * f : arg_offsets + f;
@@ -251,21 +254,41 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
   float cost[K];            // traffic of the feature in this batch (sizes tiles: 24 bits serve)
   int gran[K];              // bags per workgroup pass of the feature's schedule (kSplitGran: splits)
 
-  // Step 1, the only one that reads memory, in two rounds of loads: the addresses, the schedule
-  // and the per-lookup / per-bag bytes of every feature; then its live lookup count.
+  // Step 1, the only one that reads memory, in rounds of loads that do not wait for each other
+  // (every condition that is the same for all features stands outside the loops over them: a
+  // branch inside made the compiler wait for one feature's loads before it issued the next
+  // one's, eight round trips in a row where two do): the caller's numbers of the features (a
+  // kernel with a tile order); the addresses, the schedule and the per-lookup / per-bag bytes
+  // of every feature; then its live lookup count.  Surplus threads repeat the last feature,
+  // stores included.
   int64_t offs_at[K], idx_at[K], table_at[K];
-  int lookup_b[K], bag_b[K], cand[K];
+  int lookup_b[K], bag_b[K], cand[K], ext_f[K];
+  if (io.ext) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) ext_f[k] = io.ext[min(tid + k * BT, F - 1)];
+  } else {
+#pragma unroll
+    for (int k = 0; k < K; ++k) ext_f[k] = min(tid + k * BT, F - 1);
+  }
+  // (a model that finds its addresses per tile and gets the lookup counts needs none here)
+  if (BindingStorage<F>::kKeepAddrs || !io.counts) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) io.addrs_at(ext_f[k], idx_at[k], offs_at[k]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < K; ++k) idx_at[k] = offs_at[k] = 0;
+  }
+  // (the once-per-launch binding kernel has no use for the tables' addresses and passes none)
+  if (BindingStorage<F>::kKeepAddrs && table_ptrs) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) table_at[k] = table_ptrs[ext_f[k]];
+  } else {
+#pragma unroll
+    for (int k = 0; k < K; ++k) table_at[k] = 0;
+  }
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    // surplus threads repeat the last feature, stores included: no branch stands between the
-    // loads of this step
     const int f = min(tid + k * BT, F - 1);
-    idx_at[k] = offs_at[k] = 0;
-    // (a model that finds its addresses per tile and gets the lookup counts needs none here)
-    if (BindingStorage<F>::kKeepAddrs || !io.counts) io.addrs(f, idx_at[k], offs_at[k]);
-    table_at[k] = 0;
-    // (the once-per-launch binding kernel has no use for the tables' addresses and passes none)
-    if constexpr (BindingStorage<F>::kKeepAddrs) table_at[k] = table_ptrs ? table_ptrs[io.ext_of(f)] : 0;
     cand[k] = f;
     if constexpr (!ONE_CAND) {
       const int first = cand_begin[f];
@@ -278,6 +301,24 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     lookup_b[k] = lookup_bytes[f];
     bag_b[k] = bag_bytes[f];
   }
+  int lookups[K], first_lookup[K];
+  if (fixed_tiles) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) lookups[k] = first_lookup[k] = 0;
+  } else if (io.counts) {                     // one array for all features instead of a line each
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      lookups[k] = io.counts[ext_f[k]];
+      first_lookup[k] = 0;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int *offs = global_ptr<int>(offs_at[k]);
+      first_lookup[k] = offs[0];
+      lookups[k] = offs[B] - first_lookup[k];
+    }
+  }
   float traffic = 0.f;
 #pragma unroll
   for (int k = 0; k < K; ++k) {
@@ -286,19 +327,10 @@ bind_tiles(BindingStorage<F> &s, const IoView &io, const int tile_bytes,
     cost[k] = 0.f;
     bool one_per_bag = false;
     if (!fixed_tiles) {
-      int first_lookup = 0;
-      int lookups;
-      if (io.counts) {                        // one array for all features instead of a line each
-        lookups = io.count(f);
-      } else {
-        const int *offs = global_ptr<int>(offs_at[k]);
-        first_lookup = offs[0];
-        lookups = offs[B] - first_lookup;
-      }
-      cost[k] = static_cast<float>(lookups) * static_cast<float>(lookup_b[k]) +
+      cost[k] = static_cast<float>(lookups[k]) * static_cast<float>(lookup_b[k]) +
                 static_cast<float>(B) * static_cast<float>(bag_b[k]);
       traffic += real ? cost[k] : 0.f;
-      one_per_bag = lookups == B && first_lookup == 0;
+      one_per_bag = lookups[k] == B && first_lookup[k] == 0;
     }
     s.cand[f] = cand[k];
     if constexpr (BindingStorage<F>::kKeepAddrs) {
