@@ -217,7 +217,9 @@ def main():
 
     if args.compile_only:
         if not args.incumbent_only:
-            if tune_config.interference == "model":
+            if args.launch_only:
+                pass                    # the global stage alone needs no tuning build
+            elif tune_config.interference == "model":
                 tuner.compile_tournament(tune_config)
             else:
                 tuner.compile_local(tune_config)

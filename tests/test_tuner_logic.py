@@ -488,6 +488,29 @@ def test_incumbent_alone_goes_through_the_global_stage(tmp_path, monkeypatch):
         tuner.solve_incumbent_only(cfg._replace(incumbent=None))
 
 
+def test_schedule_transfer_adopts_unanimous_picks_by_kind():
+    """``transfer_schedule``: a kind of feature (width, type, bag-length class, default schedule)
+    takes the source's tuned pick where the source's features of that kind agree; a split vote
+    or an unknown kind keeps the default."""
+    from recflex_amd.tuning.transfer import feature_kind, transfer_schedule
+    d = lambda lanes: {"schedule": "SubWavefrontPerBagSchedule", "params": {"lanes_x": lanes}, "embed_dim": 0}
+    src_feats = [(16, "float", 8.2)] * 5 + [(32, "float", 1.0)] * 4 + [(64, "float", 40.0)] * 2
+    src_default = [d(4)] * 5 + [d(8)] * 4 + [d(16)] * 2
+    src_tuned = [d(2)] * 4 + [d(4)] + [d(8)] * 2 + [d(1)] * 2 + [d(16)] * 2     # 80 %; split; unchanged
+    dst_feats = [(16, "float", 9.9), (16, "float", 16.0), (32, "float", 1.2), (64, "float", 44.0), (16, "half", 8.0)]
+    dst_default = [d(4), d(4), d(8), d(16), d(4)]
+    out, counts = transfer_schedule(src_feats, src_default, src_tuned, dst_feats, dst_default)
+    assert [e["params"]["lanes_x"] for e in out] == [2, 4, 8, 16, 4]
+    assert counts == {"changed": 1, "kept": 1, "unknown_kind": 3}
+    assert out[0] is not dst_default[0] and dst_default[0]["params"]["lanes_x"] == 4
+    assert feature_kind(16, "float", 8.2, d(4)) == feature_kind(16, "float", 15.9, d(4))
+    assert feature_kind(16, "float", 3.4, d(4)) != feature_kind(16, "float", 3.6, d(4))
+    out, counts = transfer_schedule(src_feats, src_default, src_tuned, dst_feats, dst_default, agree=0.5)
+    assert counts == {"changed": 1, "kept": 2, "unknown_kind": 2}     # at 50 % the split vote's first pick counts
+    with pytest.raises(ValueError):
+        transfer_schedule(src_feats, src_default[:-1], src_tuned, dst_feats, dst_default)
+
+
 def test_tile_order_comes_from_the_ticks_of_the_mix_as_it_ships(tmp_path, monkeypatch):
     """The order key is ticks per tile of a timing build of the chosen mix, pooled over the
     features of one kind (schedule, parameters, row type, width): dearest kind first, features
