@@ -104,7 +104,7 @@ int recom_get_max_concurrent_blocks(int32_t *out);
  * their partial sums (entries * (36 + 16 * max dim) + 128 bytes; 4 096 entries up to 128
  * features, 16 384 beyond); a library whose last tile passes are drawn from ticket counters
  * adds those (1 152 bytes); a library that is bound once per launch (by default one of more
- * than 2048 features) adds the table into which a one-workgroup kernel binds the model (12 bytes
+ * than 3072 features) adds the table into which a one-workgroup kernel binds the model (12 bytes
  * per feature).  Replaces the
  * extra-buffer sizes the reference's host preprocessors report per batch
  * (RecFlex/code_emitter/codegen.py:149-160, extra_buffer_offsets). */
@@ -212,7 +212,7 @@ typedef struct recom_process_args {
  * and FusedKnl (RecFlex/code_emitter/codegen.py:318-383).
  * Never allocates.  A library emitted with outlier tiles (recom_info.outliers) launches a small
  * kernel ahead that walks the offsets and lists the outlier bags in the workspace.
- * A library that is bound once per launch (by default one of more than 2048 features)
+ * A library that is bound once per launch (by default one of more than 3072 features)
  * launches a one-workgroup kernel ahead of the fused one that binds the model for this batch
  * into a table in the workspace. */
 int recom_process(const recom_process_args *args);

@@ -50,14 +50,27 @@ INDEX_BYTES = 4
 # trip), expressed here as extra bytes so that tiles of narrow-row features do not run longer
 # than tiles of wide-row features.
 LOOKUP_OVERHEAD_BYTES = 0
-# Models of more features than this are bound once per launch by a small kernel instead of by
-# every workgroup of the fused kernel (rfx::bind_once), unless the emitter is told otherwise
-# (``bind_once=``).  The per-workgroup binding cannot hold more than about 2 048 features in LDS
-# beside four workgroups per CU.  Below that the two ways cost the same for the whole call:
-# measured on models of 256-bag batches of small features at four workgroups per CU, back-to-back
-# launches from a graph, per workgroup -> once per launch: 1 000 features 81.5 -> 83.8 us (the
-# fused kernel alone 82.3 -> 76.1 us, the binding kernel 7.8 us and a launch in front of it).
-BIND_ONCE_MIN_FEATS = 2048
+# Models of more features than this, or whose binding tables would not fit into LDS beside the
+# build's workgroups per CU, are bound once per launch by a small kernel instead of by every
+# workgroup of the fused kernel (rfx::bind_once), unless the emitter is told otherwise
+# (``bind_once=``).  Measured on models of 256-bag batches of small features at four workgroups
+# per CU, rotated batches, per workgroup against once per launch: 1 000 features 64.7 against
+# 69.6 us, 2 500 features 174.1 against 178.7 us (the binding kernel takes 7.2 us there and the
+# workgroups still copy the prefix array, 2.9 us; every workgroup binding for itself takes 10).
+# Before the binding's arithmetic and loads were trimmed it cost every workgroup 10 us per
+# thousand features and the limit stood at 2 048.
+BIND_ONCE_MIN_FEATS = 3072
+# LDS of a CU, and what a workgroup's binding tables take per feature (prefix, bags per tile,
+# schedule; the second level of the prefix sum) beside an allowance for the schedules' own
+LDS_BYTES_PER_CU = 160 * 1024
+BIND_LDS_ALLOWANCE = 4096
+
+
+def binds_once_by_default(num_feats: int, occupancy: int = None) -> bool:
+    if num_feats > BIND_ONCE_MIN_FEATS:
+        return True
+    tables = (num_feats + 1) * 4 + num_feats * 8 + (num_feats + 63) // 64 * 4 + 128
+    return tables + BIND_LDS_ALLOWANCE > LDS_BYTES_PER_CU // (occupancy or 4)
 # a bag becomes tiles of its own (libraries emitted with outliers=True) from this much traffic
 OUTLIER_MIN_BYTES = 128 * 1024
 
@@ -223,7 +236,7 @@ class CodeEmitter:
         flat, cand_begin = self.flat_candidates()
         embed_dim_offsets = self.embed_dim_offsets()
         if bind_once is None:
-            bind_once = num_feats > BIND_ONCE_MIN_FEATS
+            bind_once = binds_once_by_default(num_feats, occupancy)
         split_regions, workspace_floats = self.split_regions()
         has_split = workspace_floats > 0
         assert not (outliers and (timing or fixed_task_block_nums)), \
@@ -972,7 +985,7 @@ extern "C" int recom_get_feature_tables(int32_t *embed_dims, int32_t *embed_dim_
         that keeps further workgroups off the CU); ``tune`` is accepted for signature
         compatibility -- the pad is applied whenever an occupancy is given.  ``bind_once``: bind
         the model once per launch with a kernel of its own instead of in every workgroup of the
-        fused kernel (None: for models of more than BIND_ONCE_MIN_FEATS features)."""
+        fused kernel (None: ``binds_once_by_default``)."""
         code = "// generated by recflex_amd.code_emitter -- do not edit\n"
         code += self.emit_headers()
         code += self.emit_kernel(timing=timing, timing_branch=timing_branch,

@@ -293,7 +293,8 @@ def _wide(num_features: int = 1500, name: str = "wide") -> ModelSpec:
         feats.append(FeatureSpec(int(rng.integers(64, 512)), dim, "float", mean, mean == 1.0,
                                  0.0 if mean == 1.0 else 0.3, 1.05))
     wl = Workload(name, 40, num_features, tuple(feats), "integer")
-    return _default(wl)
+    # (2 500 features would fit the per-workgroup binding; ``wider`` is there for the other one)
+    return _default(wl, bind_once=True) if num_features > 2048 else _default(wl)
 
 
 def _ordered(spec: ModelSpec, name: str, seed: int, drawn_tail: int = 0, **emit_kwargs) -> ModelSpec:

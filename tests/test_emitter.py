@@ -306,3 +306,18 @@ def test_launch_bounds_carry_wavefronts_per_simd_not_workgroups_per_cu():
     fs = [default_schedule(MetaData(32, "float"), 4, 64)]
     src = CodeEmitter(fs).emit_kernel(occupancy=20)
     assert "constexpr int BLOCK_THREADS = 64;" in src and "__launch_bounds__(BLOCK_THREADS, 5)" in src
+
+
+def test_binding_once_per_launch_is_the_default_only_where_every_workgroup_cannot_bind():
+    """Up to ``BIND_ONCE_MIN_FEATS`` features every workgroup binds for itself -- unless its
+    tables (12 bytes per feature and the prefix sum's second level) would not fit into LDS beside
+    the other workgroups of the CU at the build's occupancy."""
+    from recflex_amd.code_emitter.codegen import BIND_ONCE_MIN_FEATS, binds_once_by_default
+    assert BIND_ONCE_MIN_FEATS == 3072
+    assert not binds_once_by_default(1000, 4) and not binds_once_by_default(2500, 4)
+    assert not binds_once_by_default(2500) and not binds_once_by_default(3000, 4)
+    assert binds_once_by_default(3072, 4) and not binds_once_by_default(3072, 3)     # 41 KB of LDS
+    assert binds_once_by_default(3073, 3) and binds_once_by_default(10000, 1)
+    assert binds_once_by_default(2500, 5) and not binds_once_by_default(2000, 5)
+    assert binds_once_by_default(1500, 8) and not binds_once_by_default(1000, 8)
+

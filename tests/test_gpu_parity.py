@@ -470,7 +470,7 @@ def test_every_schedule_variant_on_ragged_batches(batch, seed):
 def test_launch_replays_inside_a_hip_graph(name):
     """recom_process is a single kernel launch on the caller's stream (binding happens on the
     device, no host-side task mapping, no copies), so a serving loop can capture it once and
-    replay it (a library bound once per launch -- above 2 048 features -- launches its binding kernel first: two
+    replay it (a library bound once per launch -- by default above 3 072 features -- launches its binding kernel first: two
     kernel nodes; a library whose tiles are drawn leaves its ticket counters at zero for the next
     replay).  Captured after one eager call; replayed four times, each time with new bag
     lengths and lookups written into the same index / offset buffers, with eager work and
