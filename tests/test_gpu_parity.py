@@ -68,6 +68,20 @@ def test_binding_is_result_invariant(tile_bytes, grid, xcd):
     _assert_parity(*_run_model("c3s", tile_bytes=tile_bytes, grid_blocks=grid, xcd_segments=xcd))
 
 
+@pytest.mark.parametrize("name", ["c3s_drawn_all", "c3s_ordered"])
+@pytest.mark.parametrize("tile_bytes,grid,xcd", [(4096, 0, 0), (1 << 20, 0, 0), (0, 1, 0), (0, 7, 0),
+                                                 (16384, 96, -1), (0, 0, 1), (4096, 0, 128),
+                                                 (0, 1024, 1000), (0, 8, 3)])
+def test_drawn_walks_are_result_invariant(name, tile_bytes, grid, xcd):
+    """The same for libraries whose tiles are drawn from ticket counters (all of them; the last
+    two passes of an ordered tile space): one workgroup, grids that are not a multiple of the
+    8 XCDs (one counter for the device), more segments than tiles, fewer tiles than workgroups."""
+    wl, got, want = _run_model(name, tile_bytes=tile_bytes, grid_blocks=grid, xcd_segments=xcd)
+    assert wl.table_values == "integer"
+    bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+    assert bad.size == 0, f"{len(bad)} elements differ, first at {bad[:5].tolist()}"
+
+
 @pytest.mark.parametrize("name", ["variants", "edge", "onehots", "wide", "wider", "widest", "longbags"])
 def test_integer_tables_are_bit_exact(name):
     """Integer-valued tables make every fp32 sum exact, so each schedule variant (any lane
