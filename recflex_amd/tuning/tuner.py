@@ -1091,8 +1091,7 @@ class Tuner:
         return dirs
 
     def decide_walk(self, sched_params: List[Tuple[ScheduleBase, NamedTuple]], occupancy: int,
-                    measured_times: Dict[int, Dict[int, List[float]]], tile_bytes: int,
-                    xcd_segments: int, outliers: bool, tune_config: TuneConfig
+                    tile_bytes: int, xcd_segments: int, outliers: bool, tune_config: TuneConfig
                     ) -> Tuple[Optional[List[int]], int, int]:
         """(tile_order, drawn_tail, xcd_segments) for ``optimal/``, by measurement.
 
@@ -1190,8 +1189,7 @@ class Tuner:
             outliers = self.decide_outliers(opt_sched_params, opt_occupancy, tile_bytes, xcd_segments,
                                             tune_config)
         tile_order, drawn_tail, xcd_segments = self.decide_walk(
-            opt_sched_params, opt_occupancy, measured_times, tile_bytes, xcd_segments, bool(outliers),
-            tune_config)
+            opt_sched_params, opt_occupancy, tile_bytes, xcd_segments, bool(outliers), tune_config)
         # a contender whose library came out of the compile cache (the same source had been built
         # in another directory) has no host module of its own: optimal/ is then built in place
         import glob

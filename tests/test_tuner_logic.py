@@ -402,7 +402,6 @@ def test_tile_walk_is_decided_by_measurement(tmp_path, monkeypatch):
     workgroups get a few tiles each and an order on wide models of few tiles per workgroup."""
     tuner = _tiny_tuner(tmp_path)
     mix = [c[0] for c in tuner.feat_sched_param_candidates]
-    measured = {}
     built, times, asked = [], {}, []
     monkeypatch.setattr(Tuner, "_schedule_builds", lambda self, jobs, cfg: built.extend(j[0] for j in jobs))
     monkeypatch.setattr(Tuner, "_kernel_time", lambda self, d, cfg, mgr, tb=0, xs=0: asked.append((d, xs)))
@@ -412,14 +411,14 @@ def test_tile_walk_is_decided_by_measurement(tmp_path, monkeypatch):
     monkeypatch.setattr(Tuner, "tile_time_order", lambda self, sp, occ, tb, xs, cfg: [1, 0])
     cfg = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=1, in_process=True,
                      cluster_stage=False)
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, cfg._replace(walk_stage=False)) == (None, 0, 16)
+    assert tuner.decide_walk(mix, 4, 65536, 16, False, cfg._replace(walk_stage=False)) == (None, 0, 16)
     assert not built
     on = cfg._replace(walk_stage=True)
     names = ["as_is", "drawn_2", "drawn_4", "drawn_8", "drawn_all", "ordered", "ordered_drawn_2"]
     times.update(dict.fromkeys(names, 1000.0))
     times.update(ordered=940.0, ordered_drawn_2=900.0)
     times.update({("ordered_drawn_2", 64): 905.0, ("ordered_drawn_2", 128): 895.0})   # within the margin
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, on) == ([1, 0], 2, 16)
+    assert tuner.decide_walk(mix, 4, 65536, 16, False, on) == ([1, 0], 2, 16)
     assert [d.split("/walk_")[1].split("/")[0] for d in built] == names
     drawn = open([d for d in built if "ordered_drawn_2" in d][0] + "/process.hip").read()
     assert "#define RFX_DRAWN_TAIL 2" in drawn and "c_ext_feat" in drawn
@@ -427,35 +426,35 @@ def test_tile_walk_is_decided_by_measurement(tmp_path, monkeypatch):
     assert "#define RFX_DRAWN_TAIL 100000" in every and "c_ext_feat" not in every
     times.update(drawn_all=800.0)
     times.update({("drawn_all", 64): 790.0, ("drawn_all", 128): 700.0})
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, on) == (None, 100000, 128)
-    assert tuner.decide_walk(mix, 4, measured, 65536, 64, False, on) == (None, 100000, 128)
-    assert tuner.decide_walk(mix, 4, measured, 65536, 0, False, on) == (None, 100000, 0)    # a flat walk stays flat
+    assert tuner.decide_walk(mix, 4, 65536, 16, False, on) == (None, 100000, 128)
+    assert tuner.decide_walk(mix, 4, 65536, 64, False, on) == (None, 100000, 128)
+    assert tuner.decide_walk(mix, 4, 65536, 0, False, on) == (None, 100000, 0)    # a flat walk stays flat
     times.update(dict.fromkeys(names, 1000.0))
     times.update(ordered=995.0, drawn_8=996.0)      # within the margin
     del asked[:]
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, on) == (None, 0, 16)
+    assert tuner.decide_walk(mix, 4, 65536, 16, False, on) == (None, 0, 16)
     assert all(xs == 0 for _, xs in asked)            # no drawn winner, no finer segments timed
     del built[:]
     times.update(ordered=900.0)
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, True, on) == ([1, 0], 0, 16)
+    assert tuner.decide_walk(mix, 4, 65536, 16, True, on) == ([1, 0], 0, 16)
     assert len(built) == 2 and not any("drawn" in d for d in built)
     # left to itself: 2 features x 16 bags on 16 workgroups are less than a tile each -- nothing
     # is drawn, and the model is not wide
     del built[:]
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, cfg) == (None, 0, 16) and not built
+    assert tuner.decide_walk(mix, 4, 65536, 16, False, cfg) == (None, 0, 16) and not built
     few = cfg._replace(walk_drawn_min_tiles=0.01)
     times.update(dict.fromkeys(names, 1000.0))
     times.update(drawn_8=900.0)
     times.update({("drawn_8", 64): 950.0, ("drawn_8", 128): 960.0})
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, False, few) == (None, 8, 16)
+    assert tuner.decide_walk(mix, 4, 65536, 16, False, few) == (None, 8, 16)
     assert [d.split("/walk_")[1].split("/")[0] for d in built] == ["as_is", "drawn_2", "drawn_4", "drawn_8", "drawn_all"]
     del built[:]
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, True, few) == (None, 0, 16) and not built
+    assert tuner.decide_walk(mix, 4, 65536, 16, True, few) == (None, 0, 16) and not built
     wide = cfg._replace(walk_stage_min_feats=2, walk_stage_max_tiles=1e9)
     times.update(ordered=900.0)
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, True, wide) == ([1, 0], 0, 16)
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, True, wide._replace(walk_stage_max_tiles=0.01)) == (None, 0, 16)
-    assert tuner.decide_walk(mix, 4, measured, 65536, 16, True, wide._replace(walk_stage_min_feats=3)) == (None, 0, 16)
+    assert tuner.decide_walk(mix, 4, 65536, 16, True, wide) == ([1, 0], 0, 16)
+    assert tuner.decide_walk(mix, 4, 65536, 16, True, wide._replace(walk_stage_max_tiles=0.01)) == (None, 0, 16)
+    assert tuner.decide_walk(mix, 4, 65536, 16, True, wide._replace(walk_stage_min_feats=3)) == (None, 0, 16)
 
 
 def test_incumbent_alone_goes_through_the_global_stage(tmp_path, monkeypatch):
@@ -472,7 +471,7 @@ def test_incumbent_alone_goes_through_the_global_stage(tmp_path, monkeypatch):
     monkeypatch.setattr(Tuner, "_kernel_time", lambda self, d, cfg, mgr, tb=0, xs=0: timed.append(d))
     monkeypatch.setattr(Tuner, "_read_kernel_time", lambda self, d, cfg, tb=0, xs=0: 1000.0)
     monkeypatch.setattr(Tuner, "decide_outliers", lambda self, *a: False)
-    monkeypatch.setattr(Tuner, "decide_walk", lambda self, sp, occ, mt, tb, xs, outl, cfg: (None, 8, 64))
+    monkeypatch.setattr(Tuner, "decide_walk", lambda self, sp, occ, tb, xs, outl, cfg: (None, 8, 64))
     monkeypatch.setattr(tuner_mod, "compile_build", lambda d: None)
     cfg = TuneConfig(occupancies=[4], gpu_ids=[0], sm_count=4, num_processes=1, in_process=True,
                      incumbent=str(inc), profiler="events")
