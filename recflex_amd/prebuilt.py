@@ -530,9 +530,14 @@ def rocprof_tune_config(**overrides):
                                tile_bytes=0, **overrides)
 
 
+# what the walk stage is run with on this fixture: (occupancy, tile_bytes, xcd_segments)
+ROCPROF_FIXTURE_WALK = (5, 0, 16)
+
+
 def build_rocprof_fixture() -> str:
     """``tune_rocprof/all/o{2,5}``: the default mix as whole-model kernels, what
-    ``Tuner.tune_occupancy`` measures."""
+    ``Tuner.tune_occupancy`` measures; ``tune_rocprof/walk_*/o5``: the same mix as it is and
+    with 2 / 4 / 8 / all passes of its tile walk drawn, what ``Tuner.decide_walk`` times."""
     import multiprocessing as mp
     if mp.get_start_method(allow_none=True) != "spawn":
         mp.set_start_method("spawn", force=True)
@@ -545,6 +550,9 @@ def build_rocprof_fixture() -> str:
         if tuner._build_full(output_dir, mix, occupancy, cfg):
             jobs.append((output_dir, build_dir))
     tuner._schedule_builds(jobs, cfg)
+    occupancy, tile_bytes, xcd_segments = ROCPROF_FIXTURE_WALK
+    variants = dict({"as_is": (None, 0)}, **tuner._drawn_variants(cfg))
+    tuner._build_walk_variants(variants, mix, occupancy, tile_bytes, xcd_segments, False, cfg)
     return rocprof_fixture_dir()
 
 

@@ -61,3 +61,49 @@ def test_tune_occupancy_under_rocprofv3_agrees_with_the_events_timer():
     ratio_e = by_events[occupancies[0]] / by_events[occupancies[1]]
     assert (ratio_p > 1) == (ratio_e > 1) or abs(ratio_p - 1) < 0.1 or abs(ratio_e - 1) < 0.1
     assert abs(np.log(ratio_p / ratio_e)) < np.log(1.25), (by_profiler, by_events)
+
+
+def test_walk_stage_times_the_drawn_ends_and_every_walk_computes_the_same():
+    """``Tuner.decide_walk`` on the same model (its variants built ahead of time): the mix as it
+    is and with 2 / 4 / 8 / all passes drawn are timed, a drawn winner also with finer segments;
+    whatever it keeps is one of what it tried, and the library whose tiles are all drawn gives
+    the bits of the one whose tiles are dealt out."""
+    import torch
+    from recflex_amd import prebuilt
+    from recflex_amd.code_emitter.codegen import DRAWN_ALL
+    from recflex_amd.rec_modules import FeatEmbed
+    from recflex_amd.tuning.measure import make_table
+    d = prebuilt.rocprof_fixture_dir()
+    occupancy, tile_bytes, xcd_segments = prebuilt.ROCPROF_FIXTURE_WALK
+    libs = {name: os.path.join(d, f"walk_{name}", f"o{occupancy}", "build", "librecom.so")
+            for name in ("as_is", "drawn_2", "drawn_4", "drawn_8", "drawn_all")}
+    for lib in libs.values():
+        if not os.path.exists(lib):
+            raise RuntimeError(f"{lib} is not built: run __graft_entry__.build() first")
+    stamps = {name: os.path.getmtime(lib) for name, lib in libs.items()}
+    tuner = prebuilt.make_rocprof_tuner()
+    mix = prebuilt.fixture_default_mix(tuner)
+    print("[case] walk stage on the 100-feature fixture, events timer", flush=True)
+    cfg = prebuilt.rocprof_tune_config(profiler="events", remeasure=True, walk_drawn_min_tiles=0.0)
+    order, drawn, segments = tuner.decide_walk(mix, occupancy, tile_bytes, xcd_segments, False, cfg)
+    assert order is None                                   # a hundred features: no order is tried
+    assert drawn in (0, 2, 4, 8, DRAWN_ALL)
+    assert segments == xcd_segments or (drawn and segments in cfg.walk_xcd_segments_candidates)
+    assert stamps == {name: os.path.getmtime(lib) for name, lib in libs.items()}, "a variant was built again"
+    for name in libs:
+        t = tuner._read_kernel_time(os.path.dirname(os.path.dirname(libs[name])), cfg)
+        assert t > 0
+    dev = torch.device("cuda", 0)
+    torch.manual_seed(3)
+    tables = [make_table(shape, dtype, dev, ones=False) for shape, dtype in zip(tuner.table_shapes, tuner.data_types)]
+    idx = [torch.from_numpy(feat[0][0]).to(dev) for feat in tuner.batches]
+    off = [torch.from_numpy(feat[0][1]).to(dev) for feat in tuner.batches]
+    outs = {}
+    for name in ("as_is", "drawn_all", "drawn_2"):
+        layer = FeatEmbed(dev, embed_tables=tables, librecom=libs[name])
+        outs[name] = layer.forward_indices(idx, off).clone()
+    torch.cuda.synchronize()
+    assert not torch.isnan(outs["as_is"]).any()
+    for name in ("drawn_all", "drawn_2"):
+        assert torch.equal(outs[name].view(torch.int32), outs["as_is"].view(torch.int32)), name
+
