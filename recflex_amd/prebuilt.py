@@ -138,12 +138,18 @@ def _frozen_binding(spec: ModelSpec) -> ModelSpec:
                                [s.TileGranularity(p) for s, p in spec.feat_schedules],
                                spec.emit_kwargs.get("tile_bytes") or DEFAULT_TILE_BYTES,
                                grid_blocks=TUNE_FIXTURE_SM_COUNT * (spec.occupancy or DEFAULT_OCCUPANCY))
-    return spec._replace(emit_kwargs=dict(spec.emit_kwargs,
+    return spec._replace(emit_kwargs=dict(_plain_walk(spec.emit_kwargs),
                                           fixed_task_block_nums=[max(1, c) for c in counts]))
 
 
+def _plain_walk(emit_kwargs: dict) -> dict:
+    """The emit options without a tile order and a drawn end, which go with neither tick
+    counters nor a frozen binding nor outlier tiles."""
+    return {k: v for k, v in emit_kwargs.items() if k not in ("tile_order", "drawn_tail")}
+
+
 def _with_ticks(spec: ModelSpec) -> ModelSpec:
-    return spec._replace(emit_kwargs=dict(spec.emit_kwargs, timing=True))
+    return spec._replace(emit_kwargs=dict(_plain_walk(spec.emit_kwargs), timing=True))
 
 
 def _variants() -> ModelSpec:
@@ -252,7 +258,7 @@ def _c3_skew(outliers: bool) -> ModelSpec:
     # the schedules and launch parameters tuned for C3 (the same features; only the bag lengths
     # differ): 167 against 171 us for the default mix at five workgroups per CU, 181 at four
     spec = _tuned(wl, "c3_schedule.json")
-    return spec._replace(emit_kwargs=dict(spec.emit_kwargs, outliers=outliers))
+    return spec._replace(emit_kwargs=dict(_plain_walk(spec.emit_kwargs), outliers=outliers))
 
 
 def _few_bags(split: bool, bags: int = 16, lookups: float = 20000.0) -> ModelSpec:
