@@ -92,8 +92,8 @@ def parse_args() -> argparse.Namespace:
                              "the tile space by their time per tile, and with the last passes of the "
                              "tile walk (2, 8, all) drawn from ticket counters, and keep what is faster on the "
                              "samples; auto = a drawn end for models whose workgroups get three tiles each "
-                             "or more, an order for models of 256 features and more whose workgroups "
-                             "get fewer than eight")
+                             "or more, an order for models of 64 features and more whose workgroups "
+                             "get fewer than sixteen")
     parser.add_argument("--build_climb_trials", type=int, default=0,
                         help="global stage: that many single-feature variants of the winning mix are "
                              "built as production kernels and timed; the faster ones are adopted")

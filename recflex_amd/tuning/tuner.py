@@ -90,8 +90,8 @@ class TuneConfig(NamedTuple):
     # ``walk_stage_min_feats`` features whose workgroups get fewer than
     # ``walk_stage_max_tiles`` tiles each on the samples (with more, the deal evens out by itself)
     walk_stage: Optional[bool] = None
-    walk_stage_min_feats: int = 256
-    walk_stage_max_tiles: float = 8.0
+    walk_stage_min_feats: int = 64
+    walk_stage_max_tiles: float = 16.0
     # passes drawn at the end of the walk that are tried (DRAWN_ALL: every tile), on models whose
     # workgroups get at least ``walk_drawn_min_tiles`` tiles each on the samples
     drawn_tail_candidates: Sequence[int] = (2, 4, 8, DRAWN_ALL)
@@ -1108,7 +1108,9 @@ class Tuner:
         An order: with the features sorted by their time per tile, the strided deal hands every
         workgroup one tile of each kind, and a drawn end has cheap tiles to fill it with: 3 and
         7 % on a model of a thousand small features whose workgroups get five tiles each,
-        nothing at ten tiles per workgroup.  Tried on wide models of few tiles per workgroup.
+        1.6 % on one of a hundred features and 14 tiles per workgroup, nothing on one of 2 500
+        features and 15.  Tried on models of ``walk_stage_min_feats`` features and more whose
+        workgroups get fewer than ``walk_stage_max_tiles`` tiles.
 
         All variants are built, timed on the samples like contenders of the global stage, and
         the fastest is kept if it gains ``TuneConfig.walk_min_gain``.  A drawn winner is then
