@@ -321,3 +321,19 @@ def test_binding_once_per_launch_is_the_default_only_where_every_workgroup_canno
     assert binds_once_by_default(2500, 5) and not binds_once_by_default(2000, 5)
     assert binds_once_by_default(1500, 8) and not binds_once_by_default(1000, 8)
 
+
+
+def test_models_derived_from_a_tuned_schedule_keep_the_plain_walk_where_they_must():
+    """A tuned schedule file may carry a tile order and a drawn end; the timing build, the
+    frozen-binding build and the outlier builds made from the same file go with neither (the
+    emitter refuses the combination), so they are emitted with the plain walk."""
+    from recflex_amd import prebuilt
+    tuned = prebuilt.model_spec("c3_tuned").emit_kwargs
+    assert tuned.get("drawn_tail") and tuned.get("tile_order")
+    for name in ("c3_tuned_ticks", "c3_tuned_static", "c3_skew", "c3_skew_plain"):
+        kw = prebuilt.model_spec(name).emit_kwargs
+        assert "drawn_tail" not in kw and "tile_order" not in kw, name
+        assert kw.get("tile_bytes") == tuned.get("tile_bytes") and kw.get("xcd_segments") == tuned.get("xcd_segments")
+    for name in ("c4_tuned", "c5_tuned", "refa_tuned", "reff4_tuned"):
+        kw = prebuilt.model_spec(name).emit_kwargs
+        assert kw.get("drawn_tail", 0) > 0 and not kw.get("outliers"), name
